@@ -1,6 +1,7 @@
 """Grouped-query attention over a paged key/value cache with a per-head linear distance bias and a causal, windowed or
 chunked mask (csrc/biased_attn.hip, libhydra_mix.so):
-    score(i, j) = q_i . k_j * scale - slopes[h] * (i - j),   softmax over the keys j that position i sees.
+    score(i, j) = cap(q_i . k_j * scale) - slopes[h] * (i - j),   softmax over the keys j that position i sees,
+with cap(s) = softcap * tanh(s / softcap) when a soft cap is given and s otherwise.
 Key rows (dim) and value rows (vdim) may differ in size; a cache row holds kv_heads heads of `head_size` elements and the
 keys / values fill the first dim / vdim of each.  The caches are the pool planes [n_blocks, block_size, kv_heads, head_size]
 of the block manager; a layer with fewer heads than the pool's rows hold uses the first of each row."""
@@ -63,7 +64,7 @@ def qk_norm_cache(proj: Tensor, q_size: int, k_size: int, v_size: int, q_w: Opti
 def biased_attention(q: Tensor, key_cache: Tensor, value_cache: Tensor, vdim: int, tok_seq: Tensor, positions: Tensor,
                      q_cu: Tensor, block_table: Tensor, cu_block_lens: Tensor, scale: float,
                      slopes: Optional[Tensor] = None, mask: str = "causal", mask_size: int = 0, max_q_len: int = 0,
-                     kv_heads: Optional[int] = None, max_kv_len: int = 0, form: str = "auto") -> Tensor:
+                     kv_heads: Optional[int] = None, max_kv_len: int = 0, form: str = "auto", softcap: float = 0.0) -> Tensor:
     """q: [n_tokens, n_heads, dim] contiguous.  kv_heads: the key / value heads in use (the first of every cache row;
     default: all the plane has).  max_q_len: the longest portion of the batch; max_kv_len: the most keys a sequence holds —
     with few rows in the launch (decode steps) the keys of every tile are dealt to several waves.  form: "auto" (bfloat16
@@ -99,7 +100,7 @@ def biased_attention(q: Tensor, key_cache: Tensor, value_cache: Tensor, vdim: in
     a.cache_block_stride, a.cache_row_stride, a.head_stride, a.block_size = bstride, rstride, hstride, bs
     a.n_tokens, a.n_heads, a.kv_heads, a.dim, a.vdim = T, H, G, D, int(vdim)
     a.mask_kind, a.mask_size, a.scale, a.dtype = MASK_KINDS[mask], int(mask_size), float(scale), _code(q.dtype)
-    a.n_seq, a.max_q_len = n_seq, int(max_q_len)
+    a.n_seq, a.max_q_len, a.softcap = n_seq, int(max_q_len), float(softcap or 0.0)
     a.form, a.n_splits, a.ws_o, a.ws_ml = {"auto": 0, "rows": 1, "tile": 2}[form], 1, None, None
     if form in ("auto", "tile") and q.dtype == torch.bfloat16 and max_q_len > 0 and max_kv_len > 0 and D % 8 == 0 and vdim % 8 == 0 \
             and D <= 256 and vdim <= 256:

@@ -211,7 +211,7 @@ def lib() -> ctypes.CDLL:
 # a paged latent cache.  A library of its own, so that a model that needs only these builds only these (`make mix`).
 # ---------------------------------------------------------------------------------------------------------
 MIX_LIB_PATH = os.environ.get("HX_MIX_LIB_PATH") or os.path.join(_HERE, "lib", "libhydra_mix.so")
-HXM_ABI_VERSION = 2
+HXM_ABI_VERSION = 3
 HXM_MAX_STREAMS = 16
 HXM_MAX_LATENT = 1024
 
@@ -247,7 +247,39 @@ class hxm_biased_attn_args(ctypes.Structure):
         ("n_tokens", c_int32), ("n_heads", c_int32), ("kv_heads", c_int32), ("dim", c_int32), ("vdim", c_int32),
         ("block_size", c_int32), ("mask_kind", c_int32), ("mask_size", c_int32), ("scale", c_float), ("dtype", c_int32),
         ("q_cu", c_void_p), ("n_seq", c_int32), ("max_q_len", c_int32), ("form", c_int32), ("n_splits", c_int32),
-        ("ws_o", c_void_p), ("ws_ml", c_void_p),
+        ("ws_o", c_void_p), ("ws_ml", c_void_p), ("softcap", c_float),
+    ]
+
+
+class hxm_head_rope_args(ctypes.Structure):
+    _fields_ = [
+        ("q_out", c_void_p), ("q", c_void_p), ("k", c_void_p), ("q_stride", c_int64), ("k_stride", c_int64),
+        ("q_w", c_void_p), ("k_w", c_void_p), ("inv_freq", c_void_p), ("positions", c_void_p), ("slot_ids", c_void_p),
+        ("key_cache", c_void_p), ("value_cache", c_void_p), ("cache_row_stride", c_int64), ("head_stride", c_int64),
+        ("n_tokens", c_int64), ("q_heads", c_int32), ("kv_heads", c_int32), ("dim", c_int32), ("rot_dims", c_int32),
+        ("eps", c_float), ("cos_sin_scale", c_float), ("dtype", c_int32),
+    ]
+
+
+class hxm_state_scan_args(ctypes.Structure):
+    _fields_ = [
+        ("out", c_void_p), ("q", c_void_p), ("k", c_void_p), ("v", c_void_p),
+        ("q_stride", c_int64), ("k_stride", c_int64), ("v_stride", c_int64),
+        ("q_dtype", c_int32), ("k_dtype", c_int32), ("v_dtype", c_int32), ("decay_per_channel", c_int32),
+        ("decay", c_void_p), ("vscale", c_void_p), ("beta", c_void_p), ("bonus", c_void_p),
+        ("state", c_void_p), ("slot_stride", c_int64), ("slots", c_void_p), ("q_cu", c_void_p), ("positions", c_void_p),
+        ("n_tokens", c_int64), ("n_seq", c_int32), ("heads", c_int32), ("qk_heads", c_int32), ("dim", c_int32),
+        ("vdim", c_int32), ("mode", c_int32),
+    ]
+
+
+class hxm_group_norm_args(ctypes.Structure):
+    _fields_ = [
+        ("out", c_void_p), ("out_stride", c_int64), ("x", c_void_p), ("x_stride", c_int64), ("x_dtype", c_int32),
+        ("skip", c_void_p), ("skip_stride", c_int64), ("skip_w", c_void_p), ("skip_group", c_int32),
+        ("gate", c_void_p), ("gate_stride", c_int64), ("gate_act", c_int32), ("gate_first", c_int32),
+        ("group", c_int32), ("eps", c_float), ("w", c_void_p), ("w_len", c_int32), ("scale", c_float),
+        ("rows", c_int64), ("n", c_int64), ("dtype", c_int32),
     ]
 
 
@@ -286,6 +318,20 @@ _MIX_SIGNATURES = {
                                   c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int64, c_int,
                                   c_void_p]),
     "hxm_biased_attention": (c_int, [POINTER(hxm_biased_attn_args), c_void_p]),
+    "hxm_causal_conv": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_void_p,
+                                c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_int32, c_int, c_void_p]),
+    "hxm_token_shift_mix": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_int32, c_void_p, c_int64, c_void_p, c_void_p,
+                                    c_void_p, c_void_p, c_int64, c_int32, c_int64, c_int, c_void_p]),
+    "hxm_clamped_glu": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_float, c_float, c_float, c_int64,
+                                c_int64, c_int, c_void_p]),
+    "hxm_unary": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int64, c_int64, c_int, c_void_p]),
+    "hxm_head_gates": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
+                               c_int32, c_int, c_void_p]),
+    "hxm_decay_exp": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int, c_void_p]),
+    "hxm_unit_norm": (c_int, [c_void_p, c_void_p, c_int64, c_float, c_float, c_int64, c_int32, c_int32, c_int, c_void_p]),
+    "hxm_head_norm_rope_cache": (c_int, [POINTER(hxm_head_rope_args), c_void_p]),
+    "hxm_state_scan": (c_int, [POINTER(hxm_state_scan_args), c_void_p]),
+    "hxm_gated_group_norm": (c_int, [POINTER(hxm_group_norm_args), c_void_p]),
 }
 
 _mix = None

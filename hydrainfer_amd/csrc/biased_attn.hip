@@ -104,6 +104,9 @@ __device__ __forceinline__ void wave_lds_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// a score under a soft cap: cap * tanh(s / cap); cap 0: the score itself
+__device__ __forceinline__ float capped(float s, float cap) { return cap > 0.f ? cap * tanhf(s / cap) : s; }
+
 // the first key a query at position i sees
 __device__ __forceinline__ int first_visible(int i, int kind, int size) {
   if (kind == HXM_MASK_WINDOW) return i - size + 1 > 0 ? i - size + 1 : 0;
@@ -149,6 +152,7 @@ __global__ __launch_bounds__(256) void biased_attn_rows_kernel(hxm_biased_attn_a
       const T* kr = kc + (int64_t)table[j / BS] * a.cache_block_stride + (int64_t)(j % BS) * a.cache_row_stride;
       float dot = 0.f;
       for (int d = 0; d < D; ++d) dot += qs[d] * A::to_float(kr[d]);
+      if (a.softcap > 0.f) dot = a.softcap * tanhf(dot / a.softcap);
       s = dot - slope * (float)(i - j);
     }
     const float m_new = fmaxf(m, wave_max(s));
@@ -313,7 +317,7 @@ __global__ __launch_bounds__(256) void biased_attn_tile_kernel(hxm_biased_attn_a
       for (int s = 0; s < 2; ++s) {
         const int key = key0 + 16 * s + c;
         const bool seen = key >= lo[i] && key <= pos[i];
-        p[s] = seen ? sc[s][i] * a.scale - slope[i] * (float)(pos[i] - key) : -INFINITY;
+        p[s] = seen ? capped(sc[s][i] * a.scale, a.softcap) - slope[i] * (float)(pos[i] - key) : -INFINITY;
         mx = fmaxf(mx, p[s]);
       }
       mx = row16_max(mx);      // (the sixteen lanes that hold the row's scores: one DPP row)
@@ -518,7 +522,7 @@ __global__ __launch_bounds__(256) void biased_attn_group_kernel(hxm_biased_attn_
         for (int s = 0; s < 2; ++s) {
           const int key = key0 + 16 * s + c;
           const bool seen = key >= lo[i] && key <= pos[i];
-          p[s] = seen ? sc[s][i] * a.scale - slope[i] * (float)(pos[i] - key) : -INFINITY;
+          p[s] = seen ? capped(sc[s][i] * a.scale, a.softcap) - slope[i] * (float)(pos[i] - key) : -INFINITY;
           mx = fmaxf(mx, p[s]);
         }
         mx = row16_max(mx);

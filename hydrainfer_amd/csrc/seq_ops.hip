@@ -1,0 +1,464 @@
+// seq_ops.hip — the row kernels of mixers that keep per-sequence state beside the paged cache: short causal convolutions
+// (the inputs of the last taps - 1 positions live in the sequence's slot), token shift with several mixes (the slot
+// holds the last token's input), the clamped gated feed-forward activation, per-head decays / step sizes / write
+// strengths of a recurrence, unit norms, per-head RMS norm + rotary positions + cache append, and the gate / group norm
+// that finishes a mixer.  Everything that is not a matrix product's operand is float.
+#include "hx_common.h"
+#include "mix_rows.h"
+#include "../../include/hydra_mix.h"
+
+namespace hxm {
+int& last_hip_error();
+int check_launch();
+}  // namespace hxm
+
+namespace {
+
+using namespace hx;
+
+__device__ __forceinline__ float act_apply(float x, int act) {
+  switch (act) {
+    case HXM_ACT_SILU: return x / (1.f + expf(-x));
+    case HXM_ACT_SIGMOID: return 1.f / (1.f + expf(-x));
+    case HXM_ACT_TANH: return tanhf(x);
+    default: return x;
+  }
+}
+
+__device__ __forceinline__ float softplus(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
+
+// ------------------------------------------------------------------------------------------------ causal convolution
+template <typename A>
+__global__ __launch_bounds__(256) void causal_conv_kernel(typename A::storage* y, int64_t y_stride, const typename A::storage* u,
+                                                          int64_t u_stride, const float* w, const float* bias, int act,
+                                                          const float* state, int64_t slot_stride, const int32_t* slots,
+                                                          const int32_t* tok_seq, const int32_t* q_cu, const int32_t* positions,
+                                                          int C, int taps) {
+  const int64_t t = blockIdx.x;
+  const int seq = tok_seq[t];
+  const int64_t t0 = q_cu[seq];
+  const bool fresh = positions[t0] == 0;
+  const float* st = state + (int64_t)slots[seq] * slot_stride;
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < C; c += gridDim.y * 256) {
+    float acc = bias ? bias[c] : 0.f;
+    for (int j = 0; j < taps; ++j) {
+      const int64_t src = t - (taps - 1) + j;
+      float x = 0.f;
+      if (src >= t0) x = A::to_float(u[src * u_stride + c]);
+      else if (!fresh) x = st[(int64_t)((taps - 1) - (int)(t0 - src)) * C + c];
+      acc += w[(int64_t)c * taps + j] * x;
+    }
+    y[t * y_stride + c] = A::from_float(act_apply(acc, act));
+  }
+}
+
+// the slot afterwards: the last taps - 1 inputs of (what the slot held, then the portion); one thread a channel, ascending
+template <typename A>
+__global__ __launch_bounds__(256) void causal_conv_state_kernel(const typename A::storage* u, int64_t u_stride, float* state,
+                                                                int64_t slot_stride, const int32_t* slots, const int32_t* q_cu,
+                                                                const int32_t* positions, int C, int taps) {
+  const int seq = blockIdx.x;
+  const int64_t t0 = q_cu[seq], n = q_cu[seq + 1] - t0;
+  if (n <= 0) return;
+  const bool fresh = positions[t0] == 0;
+  float* st = state + (int64_t)slots[seq] * slot_stride;
+  const int keep = taps - 1;
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < C; c += gridDim.y * 256) {
+    for (int s = 0; s < keep; ++s) {
+      const int64_t at = n + s;                       // index into [the slot's keep entries | the portion's n inputs]
+      float x;
+      if (at >= keep) x = A::to_float(u[(t0 + at - keep) * u_stride + c]);
+      else x = fresh ? 0.f : st[(int64_t)at * C + c];
+      st[(int64_t)s * C + c] = x;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ token shift
+template <typename A>
+__global__ __launch_bounds__(256) void token_shift_mix_kernel(typename A::storage* out, const typename A::storage* h, int64_t h_stride,
+                                                              const float* mu, int n_mix, const float* state, int64_t slot_stride,
+                                                              const int32_t* slots, const int32_t* tok_seq, const int32_t* q_cu,
+                                                              const int32_t* positions, int64_t T, int64_t W) {
+  const int64_t t = blockIdx.x;
+  const int seq = tok_seq[t];
+  const int64_t t0 = q_cu[seq];
+  const bool first = t == t0, fresh = positions[t0] == 0;
+  const float* st = state + (int64_t)slots[seq] * slot_stride;
+  for (int64_t c = threadIdx.x; c < W; c += 256) {
+    const float x = A::to_float(h[t * h_stride + c]);
+    const float prev = first ? (fresh ? 0.f : st[c]) : A::to_float(h[(t - 1) * h_stride + c]);
+    const float d = prev - x;
+    for (int m = 0; m < n_mix; ++m) out[((int64_t)m * T + t) * W + c] = A::from_float(x + d * mu[(int64_t)m * W + c]);
+  }
+}
+
+template <typename A>
+__global__ __launch_bounds__(256) void token_shift_state_kernel(const typename A::storage* h, int64_t h_stride, float* state,
+                                                                int64_t slot_stride, const int32_t* slots, const int32_t* q_cu, int64_t W) {
+  const int seq = blockIdx.x;
+  const int64_t t0 = q_cu[seq], t1 = q_cu[seq + 1];
+  if (t1 <= t0) return;
+  float* st = state + (int64_t)slots[seq] * slot_stride;
+  for (int64_t c = threadIdx.x; c < W; c += 256) st[c] = A::to_float(h[(t1 - 1) * h_stride + c]);
+}
+
+// ------------------------------------------------------------------------------------------------ element-wise rows
+template <typename A>
+__global__ __launch_bounds__(256) void clamped_glu_kernel(typename A::storage* y, int64_t y_stride, const typename A::storage* gate,
+                                                          int64_t gate_stride, const typename A::storage* up, int64_t up_stride,
+                                                          float limit, float alpha, float up_shift, int64_t rows, int64_t n, int vec) {
+  if (vec) {
+    const int64_t n4 = n >> 2, total = rows * n4;
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (int64_t)gridDim.x * 256) {
+      const int64_t r = e / n4, i = (e - r * n4) * 4;
+      f32x4 g = Row4<A>::load(gate + r * gate_stride + i), u = Row4<A>::load(up + r * up_stride + i), o;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const float gg = limit > 0.f ? fminf(g[k], limit) : g[k];
+        const float uu = limit > 0.f ? fminf(fmaxf(u[k], -limit), limit) : u[k];
+        o[k] = gg / (1.f + expf(-alpha * gg)) * (uu + up_shift);
+      }
+      Row4<A>::store(y + r * y_stride + i, o);
+    }
+    return;
+  }
+  const int64_t total = rows * n;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (int64_t)gridDim.x * 256) {
+    const int64_t r = e / n, i = e - r * n;
+    const float g = A::to_float(gate[r * gate_stride + i]), u = A::to_float(up[r * up_stride + i]);
+    const float gg = limit > 0.f ? fminf(g, limit) : g;
+    const float uu = limit > 0.f ? fminf(fmaxf(u, -limit), limit) : u;
+    y[r * y_stride + i] = A::from_float(gg / (1.f + expf(-alpha * gg)) * (uu + up_shift));
+  }
+}
+
+template <typename A>
+__global__ __launch_bounds__(256) void unary_kernel(typename A::storage* out, int64_t out_stride, const typename A::storage* x,
+                                                    int64_t x_stride, int act, int64_t rows, int64_t n) {
+  const int64_t total = rows * n;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (int64_t)gridDim.x * 256) {
+    const int64_t r = e / n, i = e - r * n;
+    out[r * out_stride + i] = A::from_float(act_apply(A::to_float(x[r * x_stride + i]), act));
+  }
+}
+
+template <typename A>
+__global__ __launch_bounds__(256) void head_gates_kernel(float* decay, float* step, float* beta, const typename A::storage* a,
+                                                         int64_t a_stride, const typename A::storage* b, int64_t b_stride,
+                                                         const float* log_rate, const float* step_bias, int64_t T, int H) {
+  const int64_t total = T * H;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (int64_t)gridDim.x * 256) {
+    const int64_t t = e / H;
+    const int h = (int)(e - t * H);
+    const float sp = softplus(A::to_float(a[t * a_stride + h]) + step_bias[h]);
+    decay[e] = expf(-expf(log_rate[h]) * sp);
+    if (step) step[e] = sp;
+    if (beta) beta[e] = 1.f / (1.f + expf(-A::to_float(b[t * b_stride + h])));
+  }
+}
+
+template <typename A>
+__global__ __launch_bounds__(256) void decay_exp_kernel(float* decay, const typename A::storage* x, int64_t x_stride, const float* bias,
+                                                        int64_t rows, int64_t n) {
+  const int64_t total = rows * n;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (int64_t)gridDim.x * 256) {
+    const int64_t r = e / n, i = e - r * n;
+    decay[e] = expf(-expf(A::to_float(x[r * x_stride + i]) + (bias ? bias[i] : 0.f)));
+  }
+}
+
+// one wave per (token, head)
+template <typename A>
+__global__ __launch_bounds__(256) void unit_norm_kernel(float* out, const typename A::storage* x, int64_t x_stride, float eps, float scale,
+                                                        int64_t T, int H, int D) {
+  const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= T * H) return;
+  const int lane = threadIdx.x & 63;
+  const int64_t t = item / H;
+  const int h = (int)(item - t * H);
+  const typename A::storage* xr = x + t * x_stride + (int64_t)h * D;
+  float ss = 0.f;
+  for (int d = lane; d < D; d += 64) {
+    const float v = A::to_float(xr[d]);
+    ss += v * v;
+  }
+  ss = wave_sum(ss);
+  const float inv = scale / sqrtf(ss + eps);
+  float* o = out + (t * H + h) * D;
+  for (int d = lane; d < D; d += 64) o[d] = A::to_float(xr[d]) * inv;
+}
+
+// ------------------------------------------------------------------------------------------------ head norm + rotation + cache
+// one wave per (token, head): heads 0 .. q_heads - 1 are queries, the rest keys.  LDS: a head's normed channels per wave.
+template <typename A>
+__global__ __launch_bounds__(256) void head_norm_rope_cache_kernel(hxm_head_rope_args a) {
+  extern __shared__ float lds[];
+  typedef typename A::storage T;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int NH = a.q_heads + a.kv_heads, D = a.dim, R = a.rot_dims, half = R >> 1;
+  const int64_t item = (int64_t)blockIdx.x * 4 + wave;
+  if (item >= a.n_tokens * NH) return;
+  const int64_t t = item / NH;
+  const int h = (int)(item - t * NH);
+  const bool is_q = h < a.q_heads;
+  const int g = is_q ? h : h - a.q_heads;
+  const T* x = is_q ? (const T*)a.q + t * a.q_stride + (int64_t)g * D : (const T*)a.k + t * a.k_stride + (int64_t)g * D;
+  const float* w = is_q ? a.q_w : a.k_w;
+  float* nb = lds + wave * D;
+  T* vrow = nullptr;
+  T* orow;
+  if (is_q) {
+    orow = (T*)a.q_out + (t * a.q_heads + g) * D;
+  } else {
+    const int64_t slot = a.slot_ids[t];
+    orow = (T*)a.key_cache + slot * a.cache_row_stride + (int64_t)g * a.head_stride;
+    vrow = (T*)a.value_cache + slot * a.cache_row_stride + (int64_t)g * a.head_stride;
+  }
+  float ss = 0.f;
+  for (int d = lane; d < D; d += 64) {
+    const T raw = x[d];
+    const float v = A::to_float(raw);
+    if (vrow) vrow[d] = raw;
+    ss += v * v;
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)D + a.eps);
+  for (int d = lane; d < D; d += 64) nb[d] = A::to_float(x[d]) * inv * w[d];
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const float p = (float)a.positions[t];
+  for (int d = lane; d < D; d += 64) {
+    float o = nb[d];
+    if (d < R) {
+      const int i = d < half ? d : d - half;
+      float sn, cs;
+      sincosf(p * a.inv_freq[i], &sn, &cs);
+      sn *= a.cos_sin_scale;
+      cs *= a.cos_sin_scale;
+      o = d < half ? nb[d] * cs - nb[d + half] * sn : nb[d] * cs + nb[d - half] * sn;
+    }
+    orow[d] = A::from_float(o);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ gate / group norm
+template <typename A, typename X>
+__device__ __forceinline__ float gn_value(const hxm_group_norm_args& a, int64_t r, int64_t c) {
+  float v = X::to_float(((const typename X::storage*)a.x)[r * a.x_stride + c]);
+  if (a.skip) v += a.skip_w[c / a.skip_group] * A::to_float(((const typename A::storage*)a.skip)[r * a.skip_stride + c]);
+  if (a.gate && a.gate_first) v *= act_apply(A::to_float(((const typename A::storage*)a.gate)[r * a.gate_stride + c]), a.gate_act);
+  return v;
+}
+
+// one wave per (row, group): the group's sum of squares, then the elements once more
+template <typename A, typename X>
+__global__ __launch_bounds__(256) void gated_group_norm_kernel(hxm_group_norm_args a) {
+  typedef typename A::storage T;
+  const int lane = threadIdx.x & 63;
+  const int64_t gs = a.group > 0 ? a.group : (a.n < 1024 ? a.n : 1024);        // no norm: the groups only deal the work
+  const int64_t n_groups = (a.n + gs - 1) / gs;
+  const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= a.rows * n_groups) return;
+  const int64_t r = item / n_groups, c0 = (item - r * n_groups) * gs;
+  const int64_t c1 = c0 + gs < a.n ? c0 + gs : a.n;
+  float inv = 1.f;
+  if (a.group > 0) {
+    float ss = 0.f;
+    for (int64_t c = c0 + lane; c < c1; c += 64) {
+      const float v = gn_value<A, X>(a, r, c);
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    inv = 1.0f / sqrtf(ss / (float)gs + a.eps);
+  }
+  T* o = (T*)a.out + r * a.out_stride;
+  for (int64_t c = c0 + lane; c < c1; c += 64) {
+    float v = gn_value<A, X>(a, r, c) * inv;
+    if (a.w) v *= a.w[c % a.w_len];
+    if (a.gate && !a.gate_first) v *= act_apply(A::to_float(((const T*)a.gate)[r * a.gate_stride + c]), a.gate_act);
+    o[c] = A::from_float(v * a.scale);
+  }
+}
+
+inline unsigned flat_blocks(int64_t total) {
+  const int64_t b = (total + 255) / 256;
+  return (unsigned)(b < 1 ? 1 : (b > 16384 ? 16384 : b));
+}
+
+}  // namespace
+
+#define HXM_BY_DTYPE(dtype, CALL_F32, CALL_BF16) \
+  switch (dtype) {                               \
+    case HX_F32: CALL_F32; break;                \
+    case HX_BF16: CALL_BF16; break;              \
+    default: return HX_ERR_DTYPE;                \
+  }
+
+extern "C" int hxm_causal_conv(void* y, int64_t y_stride, const void* u, int64_t u_stride, const float* w, const float* bias, int act,
+                               float* state, int64_t slot_stride, const int32_t* slots, const int32_t* tok_seq, const int32_t* q_cu,
+                               const int32_t* positions, int64_t n_tokens, int32_t n_seq, int32_t channels, int32_t taps, int dtype,
+                               void* stream) {
+  if (n_tokens < 0 || n_seq < 0 || channels < 1 || taps < 1) return HX_ERR_SHAPE;
+  if (n_tokens == 0 || n_seq == 0) return HX_OK;
+  if (!y || !u || !w || !state || !slots || !tok_seq || !q_cu || !positions) return HX_ERR_NULL;
+  if (y_stride < channels || u_stride < channels) return HX_ERR_STRIDE;
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned cb = (unsigned)((channels + 255) / 256);
+  const dim3 grid((unsigned)n_tokens, cb < 64 ? cb : 64), sgrid((unsigned)n_seq, cb < 64 ? cb : 64), block(256);
+  HXM_BY_DTYPE(dtype,
+               (causal_conv_kernel<F32><<<grid, block, 0, s>>>((float*)y, y_stride, (const float*)u, u_stride, w, bias, act, state, slot_stride,
+                                                               slots, tok_seq, q_cu, positions, channels, taps)),
+               (causal_conv_kernel<BF16><<<grid, block, 0, s>>>((u16*)y, y_stride, (const u16*)u, u_stride, w, bias, act, state, slot_stride,
+                                                                slots, tok_seq, q_cu, positions, channels, taps)))
+  int rc = hxm::check_launch();
+  if (rc != HX_OK || taps == 1) return rc;
+  HXM_BY_DTYPE(dtype,
+               (causal_conv_state_kernel<F32><<<sgrid, block, 0, s>>>((const float*)u, u_stride, state, slot_stride, slots, q_cu, positions,
+                                                                      channels, taps)),
+               (causal_conv_state_kernel<BF16><<<sgrid, block, 0, s>>>((const u16*)u, u_stride, state, slot_stride, slots, q_cu, positions,
+                                                                       channels, taps)))
+  return hxm::check_launch();
+}
+
+extern "C" int hxm_token_shift_mix(void* out, const void* h, int64_t h_stride, const float* mu, int32_t n_mix, float* state,
+                                   int64_t slot_stride, const int32_t* slots, const int32_t* tok_seq, const int32_t* q_cu,
+                                   const int32_t* positions, int64_t n_tokens, int32_t n_seq, int64_t width, int dtype, void* stream) {
+  if (n_tokens < 0 || n_seq < 0 || width < 1 || n_mix < 1) return HX_ERR_SHAPE;
+  if (n_tokens == 0 || n_seq == 0) return HX_OK;
+  if (!out || !h || !mu || !state || !slots || !tok_seq || !q_cu || !positions) return HX_ERR_NULL;
+  if (h_stride < width) return HX_ERR_STRIDE;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)n_tokens), sgrid((unsigned)n_seq), block(256);
+  HXM_BY_DTYPE(dtype,
+               (token_shift_mix_kernel<F32><<<grid, block, 0, s>>>((float*)out, (const float*)h, h_stride, mu, n_mix, state, slot_stride, slots,
+                                                                   tok_seq, q_cu, positions, n_tokens, width)),
+               (token_shift_mix_kernel<BF16><<<grid, block, 0, s>>>((u16*)out, (const u16*)h, h_stride, mu, n_mix, state, slot_stride, slots,
+                                                                    tok_seq, q_cu, positions, n_tokens, width)))
+  int rc = hxm::check_launch();
+  if (rc != HX_OK) return rc;
+  HXM_BY_DTYPE(dtype,
+               (token_shift_state_kernel<F32><<<sgrid, block, 0, s>>>((const float*)h, h_stride, state, slot_stride, slots, q_cu, width)),
+               (token_shift_state_kernel<BF16><<<sgrid, block, 0, s>>>((const u16*)h, h_stride, state, slot_stride, slots, q_cu, width)))
+  return hxm::check_launch();
+}
+
+extern "C" int hxm_clamped_glu(void* y, int64_t y_stride, const void* gate, int64_t gate_stride, const void* up, int64_t up_stride,
+                               float limit, float alpha, float up_shift, int64_t rows, int64_t n, int dtype, void* stream) {
+  if (rows < 0 || n < 1) return HX_ERR_SHAPE;
+  if (rows == 0) return HX_OK;
+  if (!y || !gate || !up) return HX_ERR_NULL;
+  if (y_stride < n || gate_stride < n || up_stride < n) return HX_ERR_STRIDE;
+  hipStream_t s = (hipStream_t)stream;
+  const uintptr_t es = dtype == HX_F32 ? 4 : 2;
+  const int vec = n % 4 == 0 && y_stride % 4 == 0 && gate_stride % 4 == 0 && up_stride % 4 == 0 && (uintptr_t)y % (4 * es) == 0 &&
+                  (uintptr_t)gate % (4 * es) == 0 && (uintptr_t)up % (4 * es) == 0;
+  const dim3 grid(flat_blocks(vec ? rows * n / 4 : rows * n)), block(256);
+  HXM_BY_DTYPE(dtype,
+               (clamped_glu_kernel<F32><<<grid, block, 0, s>>>((float*)y, y_stride, (const float*)gate, gate_stride, (const float*)up, up_stride,
+                                                               limit, alpha, up_shift, rows, n, vec)),
+               (clamped_glu_kernel<BF16><<<grid, block, 0, s>>>((u16*)y, y_stride, (const u16*)gate, gate_stride, (const u16*)up, up_stride,
+                                                                limit, alpha, up_shift, rows, n, vec)))
+  return hxm::check_launch();
+}
+
+extern "C" int hxm_unary(void* out, int64_t out_stride, const void* x, int64_t x_stride, int act, int64_t rows, int64_t n, int dtype,
+                         void* stream) {
+  if (rows < 0 || n < 1) return HX_ERR_SHAPE;
+  if (rows == 0) return HX_OK;
+  if (!out || !x) return HX_ERR_NULL;
+  if (out_stride < n || x_stride < n) return HX_ERR_STRIDE;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid(flat_blocks(rows * n)), block(256);
+  HXM_BY_DTYPE(dtype, (unary_kernel<F32><<<grid, block, 0, s>>>((float*)out, out_stride, (const float*)x, x_stride, act, rows, n)),
+               (unary_kernel<BF16><<<grid, block, 0, s>>>((u16*)out, out_stride, (const u16*)x, x_stride, act, rows, n)))
+  return hxm::check_launch();
+}
+
+extern "C" int hxm_head_gates(float* decay, float* step, float* beta, const void* a, int64_t a_stride, const void* b, int64_t b_stride,
+                              const float* log_rate, const float* step_bias, int64_t n_tokens, int32_t heads, int dtype, void* stream) {
+  if (n_tokens < 0 || heads < 1) return HX_ERR_SHAPE;
+  if (n_tokens == 0) return HX_OK;
+  if (!decay || !a || !log_rate || !step_bias || (beta && !b)) return HX_ERR_NULL;
+  if (a_stride < heads || (b && b_stride < heads)) return HX_ERR_STRIDE;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid(flat_blocks(n_tokens * heads)), block(256);
+  HXM_BY_DTYPE(dtype,
+               (head_gates_kernel<F32><<<grid, block, 0, s>>>(decay, step, beta, (const float*)a, a_stride, (const float*)b, b_stride, log_rate,
+                                                              step_bias, n_tokens, heads)),
+               (head_gates_kernel<BF16><<<grid, block, 0, s>>>(decay, step, beta, (const u16*)a, a_stride, (const u16*)b, b_stride, log_rate,
+                                                               step_bias, n_tokens, heads)))
+  return hxm::check_launch();
+}
+
+extern "C" int hxm_decay_exp(float* decay, const void* x, int64_t x_stride, const float* bias, int64_t rows, int64_t n, int dtype,
+                             void* stream) {
+  if (rows < 0 || n < 1) return HX_ERR_SHAPE;
+  if (rows == 0) return HX_OK;
+  if (!decay || !x) return HX_ERR_NULL;
+  if (x_stride < n) return HX_ERR_STRIDE;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid(flat_blocks(rows * n)), block(256);
+  HXM_BY_DTYPE(dtype, (decay_exp_kernel<F32><<<grid, block, 0, s>>>(decay, (const float*)x, x_stride, bias, rows, n)),
+               (decay_exp_kernel<BF16><<<grid, block, 0, s>>>(decay, (const u16*)x, x_stride, bias, rows, n)))
+  return hxm::check_launch();
+}
+
+extern "C" int hxm_unit_norm(float* out, const void* x, int64_t x_stride, float eps, float scale, int64_t n_tokens, int32_t heads,
+                             int32_t dim, int dtype, void* stream) {
+  if (n_tokens < 0 || heads < 1 || dim < 1) return HX_ERR_SHAPE;
+  if (n_tokens == 0) return HX_OK;
+  if (!out || !x) return HX_ERR_NULL;
+  if (x_stride < (int64_t)heads * dim) return HX_ERR_STRIDE;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)((n_tokens * heads + 3) / 4)), block(256);
+  HXM_BY_DTYPE(dtype, (unit_norm_kernel<F32><<<grid, block, 0, s>>>(out, (const float*)x, x_stride, eps, scale, n_tokens, heads, dim)),
+               (unit_norm_kernel<BF16><<<grid, block, 0, s>>>(out, (const u16*)x, x_stride, eps, scale, n_tokens, heads, dim)))
+  return hxm::check_launch();
+}
+
+extern "C" int hxm_head_norm_rope_cache(const hxm_head_rope_args* args, void* stream) {
+  if (!args) return HX_ERR_NULL;
+  const hxm_head_rope_args& a = *args;
+  if (a.n_tokens < 0 || a.q_heads < 0 || a.kv_heads < 0 || a.q_heads + a.kv_heads < 1 || a.dim < 1 || a.rot_dims < 0 || a.rot_dims > a.dim ||
+      (a.rot_dims & 1))
+    return HX_ERR_SHAPE;
+  if (a.n_tokens == 0) return HX_OK;
+  if (!a.positions || (a.rot_dims && !a.inv_freq)) return HX_ERR_NULL;
+  if (a.q_heads && (!a.q || !a.q_out || !a.q_w)) return HX_ERR_NULL;
+  if (a.kv_heads && (!a.k || !a.k_w || !a.slot_ids || !a.key_cache || !a.value_cache)) return HX_ERR_NULL;
+  if ((a.q_heads && a.q_stride < (int64_t)a.q_heads * a.dim) || (a.kv_heads && a.k_stride < (int64_t)a.kv_heads * a.dim)) return HX_ERR_STRIDE;
+  if (a.kv_heads && (a.head_stride < a.dim || a.cache_row_stride < a.head_stride * a.kv_heads)) return HX_ERR_STRIDE;
+  const size_t lds = 4 * (size_t)a.dim * sizeof(float);
+  if (lds > 64 * 1024) return HX_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)((a.n_tokens * (a.q_heads + a.kv_heads) + 3) / 4)), block(256);
+  HXM_BY_DTYPE(a.dtype, (head_norm_rope_cache_kernel<F32><<<grid, block, lds, s>>>(a)),
+               (head_norm_rope_cache_kernel<BF16><<<grid, block, lds, s>>>(a)))
+  return hxm::check_launch();
+}
+
+extern "C" int hxm_gated_group_norm(const hxm_group_norm_args* args, void* stream) {
+  if (!args) return HX_ERR_NULL;
+  const hxm_group_norm_args& a = *args;
+  if (a.rows < 0 || a.n < 1 || a.group < 0 || (a.group > 0 && a.n % a.group) || (a.w && a.w_len < 1) || (a.skip && a.skip_group < 1))
+    return HX_ERR_SHAPE;
+  if (a.rows == 0) return HX_OK;
+  if (!a.out || !a.x || (a.skip && !a.skip_w)) return HX_ERR_NULL;
+  if (a.out_stride < a.n || a.x_stride < a.n || (a.skip && a.skip_stride < a.n) || (a.gate && a.gate_stride < a.n)) return HX_ERR_STRIDE;
+  if (a.x_dtype != HX_F32 && a.x_dtype != a.dtype) return HX_ERR_DTYPE;
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t gs = a.group > 0 ? a.group : (a.n < 1024 ? a.n : 1024);
+  const int64_t items = a.rows * ((a.n + gs - 1) / gs);
+  const dim3 grid((unsigned)((items + 3) / 4)), block(256);
+  if (a.dtype == HX_F32) {
+    gated_group_norm_kernel<F32, F32><<<grid, block, 0, s>>>(a);
+  } else if (a.dtype == HX_BF16) {
+    if (a.x_dtype == HX_F32) gated_group_norm_kernel<BF16, F32><<<grid, block, 0, s>>>(a);
+    else gated_group_norm_kernel<BF16, BF16><<<grid, block, 0, s>>>(a);
+  } else {
+    return HX_ERR_DTYPE;
+  }
+  return hxm::check_launch();
+}

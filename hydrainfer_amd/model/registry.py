@@ -60,6 +60,16 @@ def _load_kezolix(model_path: str, dtype, device, **_):
     return TextLanguageModel(model), None
 
 
+def _load_fasanex(model_path: str, dtype, device, **_):
+    from hydrainfer_amd.model.fasanex import FasanexForCausalLM, read_shape
+    from hydrainfer_amd.model.llava import TextLanguageModel
+    from hydrainfer_amd.model.loader import scan_safetensors
+    shape = read_shape(model_path)
+    model = FasanexForCausalLM.from_state_dict(shape, scan_safetensors(model_path, ("",)), dtype, device)
+    return TextLanguageModel(model), None
+
+
 register("LlavaForConditionalGeneration", _load_llava)
 register("Tetepel", _load_tetepel)
 register("Kezolix", _load_kezolix)
+register("Fasanex", _load_fasanex)

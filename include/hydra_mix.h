@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define HXM_ABI_VERSION 2
+#define HXM_ABI_VERSION 3
 #define HXM_MAX_STREAMS 16
 #define HXM_MAX_LATENT 1024     /* widest latent row the attention kernels hold in registers (the MFMA tile form: 512) */
 
@@ -246,11 +246,144 @@ typedef struct hxm_biased_attn_args {
   int32_t n_splits;          /* tile form, > 1: a tile's keys are dealt to n_splits waves (<= 64) and merged by a second kernel */
   float* ws_o;               /* n_splits > 1: n_seq * kv_heads * ceil(max_q_len * heads / kv_heads / 16) * n_splits * 16 * ceil16(vdim) floats */
   float* ws_ml;              /* n_splits > 1: ... * n_splits * 32 floats */
+  float softcap;             /* > 0: q . k * scale becomes softcap * tanh(q . k * scale / softcap) before the bias; 0: none */
 } hxm_biased_attn_args;
 
 /* Softmax attention of every query over the keys of its own sequence that its mask lets it see (scores and weights in
  * float).  Queries of portions and single decoded tokens may share a batch. */
 int hxm_biased_attention(const hxm_biased_attn_args* args, void* stream);
+
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * Sequence mixers with per-sequence state beside the paged cache (csrc/seq_ops.hip, csrc/state_scan.hip): short causal
+ * convolutions, token shift with several mixes, per-head norm + rotary positions + cache append, decays and step sizes
+ * of recurrences, a scan over a matrix state per head (decayed sum, read-before-write with a bonus, delta rule), and the
+ * gate / group norm that finishes a mixer.  A sequence's state lives in its state slot: `state` points at the piece's
+ * first float in slot 0, slot s is slot_stride floats further.  A portion whose first position is 0 starts from zeros
+ * without reading its slot.  q_cu [n_seq + 1]: the batch's portions; positions [n_tokens]; slots [n_seq].
+ * ------------------------------------------------------------------------------------------------------------------ */
+
+#define HXM_ACT_NONE 0
+#define HXM_ACT_SILU 1
+#define HXM_ACT_SIGMOID 2
+#define HXM_ACT_TANH 3
+
+/* y[t, c] = act(sum_j w[c, j] u[t - taps + 1 + j, c] + bias[c]) over each sequence, zeros before position 0; the inputs
+ * of the taps - 1 positions before a portion come from the slot ([taps - 1, channels] floats, oldest first), which is
+ * then brought up to date.  u, y: dtype rows; w: float [channels, taps]; bias: float [channels] or NULL. */
+int hxm_causal_conv(void* y, int64_t y_stride, const void* u, int64_t u_stride, const float* w, const float* bias, int act,
+                    float* state, int64_t slot_stride, const int32_t* slots, const int32_t* tok_seq, const int32_t* q_cu,
+                    const int32_t* positions, int64_t n_tokens, int32_t n_seq, int32_t channels, int32_t taps, int dtype,
+                    void* stream);
+
+/* out[m, t, :] = h[t] + (h[t - 1] - h[t]) * mu[m] for m < n_mix, h[t - 1] of the same sequence (zeros before position 0;
+ * across portions through the slot's `width` floats, left holding the portion's last h).  h: dtype [n_tokens, width]
+ * rows; mu: float [n_mix, width]; out: dtype [n_mix, n_tokens, width] contiguous. */
+int hxm_token_shift_mix(void* out, const void* h, int64_t h_stride, const float* mu, int32_t n_mix, float* state,
+                        int64_t slot_stride, const int32_t* slots, const int32_t* tok_seq, const int32_t* q_cu,
+                        const int32_t* positions, int64_t n_tokens, int32_t n_seq, int64_t width, int dtype, void* stream);
+
+/* y = g * sigmoid(alpha * g) * (u + up_shift) with g = min(gate, limit), u = clamp(up, -limit, limit) (limit <= 0: no
+ * clamp).  gate, up: dtype rows (two halves of one projection will do); y: dtype [rows, n]. */
+int hxm_clamped_glu(void* y, int64_t y_stride, const void* gate, int64_t gate_stride, const void* up, int64_t up_stride,
+                    float limit, float alpha, float up_shift, int64_t rows, int64_t n, int dtype, void* stream);
+
+/* out = act(x) element by element (HXM_ACT_*), dtype rows. */
+int hxm_unary(void* out, int64_t out_stride, const void* x, int64_t x_stride, int act, int64_t rows, int64_t n, int dtype,
+              void* stream);
+
+/* Per token and head, in float: step = softplus(a[t, h] + step_bias[h]), decay = exp(-exp(log_rate[h]) * step),
+ * beta = sigmoid(b[t, h]).  a, b: dtype rows (b NULL: no beta); decay, step, beta: float [n_tokens, heads] (step / beta
+ * NULL: not wanted). */
+int hxm_head_gates(float* decay, float* step, float* beta, const void* a, int64_t a_stride, const void* b, int64_t b_stride,
+                   const float* log_rate, const float* step_bias, int64_t n_tokens, int32_t heads, int dtype, void* stream);
+
+/* decay[t, c] = exp(-exp(x[t, c] + bias[c])) in float.  x: dtype rows; bias: float [n] or NULL; decay: float [rows, n]. */
+int hxm_decay_exp(float* decay, const void* x, int64_t x_stride, const float* bias, int64_t rows, int64_t n, int dtype,
+                  void* stream);
+
+/* out[t, h, :] = x[t, h, :] / sqrt(sum(x[t, h, :]^2) + eps) * scale in float.  x: dtype rows of heads * dim; out: float
+ * [n_tokens, heads * dim]. */
+int hxm_unit_norm(float* out, const void* x, int64_t x_stride, float eps, float scale, int64_t n_tokens, int32_t heads,
+                  int32_t dim, int dtype, void* stream);
+
+typedef struct hxm_head_rope_args {
+  void* q_out;               /* dtype [n_tokens, q_heads * dim] contiguous */
+  const void* q;             /* dtype rows of q_heads * dim */
+  const void* k;             /* dtype rows of kv_heads * dim */
+  int64_t q_stride, k_stride;
+  const float* q_w;          /* [dim]: weight of the per-head RMS norm, shared by the heads */
+  const float* k_w;
+  const float* inv_freq;     /* [rot_dims / 2]: angle of pair i at position p = p * inv_freq[i]; channel i turns with i + rot_dims / 2 */
+  const int32_t* positions;  /* [n_tokens] */
+  const int32_t* slot_ids;   /* [n_tokens]: cache row of every token (block * block_size + row) */
+  void* key_cache;           /* normed and turned keys go here, */
+  void* value_cache;         /* the keys as they came (before norm and rotation) here: the layer's values */
+  int64_t cache_row_stride, head_stride;
+  int64_t n_tokens;
+  int32_t q_heads, kv_heads, dim, rot_dims;
+  float eps, cos_sin_scale;  /* cos and sin are multiplied by cos_sin_scale */
+  int32_t dtype;
+} hxm_head_rope_args;
+
+/* Per-head RMS norm (plain weight) of queries and keys, rotary positions on the first rot_dims channels of every head
+ * (angles, cos and sin in float), keys and values appended to the paged cache. */
+int hxm_head_norm_rope_cache(const hxm_head_rope_args* args, void* stream);
+
+#define HXM_SCAN_DECAY 0      /* S <- a S + k (s v)^T;  o = S^T q */
+#define HXM_SCAN_BONUS 1      /* o = (S + diag(u) k v^T)^T q;  then S <- a S + k v^T */
+#define HXM_SCAN_DELTA 2      /* S <- a S;  S <- S + k (b (v - S^T k))^T;  o = S^T q */
+
+typedef struct hxm_state_scan_args {
+  float* out;                /* float [n_tokens, heads * vdim] contiguous */
+  const void* q;             /* rows of qk_heads * dim; head h reads q / k head h / (heads / qk_heads) */
+  const void* k;
+  const void* v;             /* rows of heads * vdim */
+  int64_t q_stride, k_stride, v_stride;
+  int32_t q_dtype, k_dtype, v_dtype;     /* HX_F32 or HX_BF16, each operand its own */
+  int32_t decay_per_channel; /* 0: decay float [n_tokens, heads]; 1: float [n_tokens, heads * dim] (a: one per key channel) */
+  const float* decay;
+  const float* vscale;       /* float [n_tokens, heads] or NULL: s above (HXM_SCAN_DECAY) */
+  const float* beta;         /* float [n_tokens, heads]: b above (HXM_SCAN_DELTA) */
+  const float* bonus;        /* float [heads * dim]: u above (HXM_SCAN_BONUS) */
+  float* state;              /* the piece [heads, dim, vdim] of every slot */
+  int64_t slot_stride;
+  const int32_t* slots;
+  const int32_t* q_cu;
+  const int32_t* positions;
+  int64_t n_tokens;
+  int32_t n_seq, heads, qk_heads, dim, vdim, mode;
+} hxm_state_scan_args;
+
+/* The recurrence of one matrix state S [dim, vdim] per head and sequence, token by token in float, continued from and
+ * left in the sequence's slot.  dim <= 256. */
+int hxm_state_scan(const hxm_state_scan_args* args, void* stream);
+
+typedef struct hxm_group_norm_args {
+  void* out;                 /* dtype rows of n */
+  int64_t out_stride;
+  const void* x;             /* x_dtype rows of n */
+  int64_t x_stride;
+  int32_t x_dtype;
+  const void* skip;          /* dtype rows of n or NULL: x += skip_w[c / skip_group] * skip */
+  int64_t skip_stride;
+  const float* skip_w;
+  int32_t skip_group;
+  const void* gate;          /* dtype rows of n or NULL */
+  int64_t gate_stride;
+  int32_t gate_act;          /* HXM_ACT_* */
+  int32_t gate_first;        /* 1: x *= act(gate) before the norm; 0: after it */
+  int32_t group;             /* > 0: every `group` consecutive elements are divided by their root mean square; 0: no norm */
+  float eps;
+  const float* w;            /* float [w_len] or NULL: element c is multiplied by w[c % w_len] after the norm */
+  int32_t w_len;
+  float scale;               /* the result is multiplied by scale */
+  int64_t rows, n;
+  int32_t dtype;
+} hxm_group_norm_args;
+
+/* What finishes a mixer: out = scale * [act(gate)] * w * rms_div_groups(x + skip_w * skip [* act(gate)]), in float. */
+int hxm_gated_group_norm(const hxm_group_norm_args* args, void* stream);
 
 
 #ifdef __cplusplus
