@@ -110,7 +110,7 @@ class MixerSpec:
 @dataclass
 class FeedForwardSpec:
     ff: int
-    limit: float = 0.0
+    limit: Optional[float] = None     # None: gate and up are not clamped
 
 
 @dataclass
@@ -226,7 +226,7 @@ class FasanexShape:
             if mlp is not None:
                 if mlp.get("kind", "dense") != "dense":
                     raise ValueError(f"layer {i}: unknown feed-forward kind {mlp['kind']!r}")
-                spec = FeedForwardSpec(int(mlp["ff"]), float(mlp.get("limit") or 0.0))
+                spec = FeedForwardSpec(int(mlp["ff"]), float(mlp["limit"]) if mlp.get("limit") is not None else None)
             layers.append(FasanexLayer(mixer, spec))
         return cls(vocab_size=int(cfg["vocab"]), hidden_size=int(cfg["width"]), layers=layers,
                    norm_eps=float((cfg.get("norm") or {}).get("eps", 1e-5)),
@@ -255,7 +255,9 @@ class FasanexShape:
                          "right": {"dim": r.dim, "heads": r.heads, "decay_rank": r.decay_rank}}
             else:
                 mixer = {"conv": m.conv, "dim": m.dim, "heads": m.heads, "kv_heads": m.kv_heads, "vdim": m.vdim}
-            mlp = None if l.mlp is None else {"kind": "dense", "ff": l.mlp.ff, "limit": l.mlp.limit}
+            mlp = None if l.mlp is None else {"kind": "dense", "ff": l.mlp.ff}
+            if mlp is not None and l.mlp.limit is not None:
+                mlp["limit"] = l.mlp.limit
             out.append({"type": m.type, "mixer": mixer, "mlp": mlp})
         return {"architecture": ARCHITECTURE, "vocab": self.vocab_size, "width": self.hidden_size,
                 "norm": {"eps": self.norm_eps}, "embedding": {"scale": self.embedding_scale}, "layers": out}
@@ -490,7 +492,7 @@ class FasanexForCausalLM:
     def _feed_forward(self, i: int, h: Tensor) -> Tensor:
         f, w = self.shape.layers[i].mlp, self.lw[i]
         gu = torch.matmul(h, w.gate_up.t())
-        return torch.matmul(clamped_glu(gu[:, :f.ff], gu[:, f.ff:], f.limit, GLU_ALPHA, 1.0), w.down.t())
+        return torch.matmul(clamped_glu(gu[:, :f.ff], gu[:, f.ff:], f.limit if f.limit is not None else 0.0, GLU_ALPHA, 1.0), w.down.t())
 
     # ------------------------------------------------------------------ forward
     def forward_hidden(self, input_ids: Tensor, position_ids: Tensor, model_params) -> Tensor:

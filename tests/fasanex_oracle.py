@@ -93,15 +93,19 @@ def window_attention(h: torch.Tensor, W: Dict[str, torch.Tensor], p: str, m: dic
     k = short_conv(h @ W[p + "k"].T, W[p + "k.conv"]).reshape(n, G, D)
     v = k                                                     # values: the keys before norm and rotation
     pos = torch.arange(n)
-    q = rotate(rms_div(q, eps) * W[p + "q.norm"], pos, m["rot"])
-    k = rotate(rms_div(k, eps) * W[p + "k.norm"], pos, m["rot"])
+    q, k = rms_div(q, eps) * W[p + "q.norm"], rms_div(k, eps) * W[p + "k.norm"]
+    if m.get("rot"):
+        q, k = rotate(q, pos, m["rot"]), rotate(k, pos, m["rot"])
     i, j = pos[:, None], pos[None, :]
-    see = (j <= i) & (i - j < m["mask"]["size"])
+    see = j <= i
+    if m.get("mask"):
+        see = see & (i - j < m["mask"]["size"])
     out = torch.zeros(n, H, v.shape[-1], dtype=F)
     for hd in range(H):
         g = hd // (H // G)
         s = (q[:, hd] @ k[:, g].T) * m["scale"]
-        s = m["softcap"] * torch.tanh(s / m["softcap"])
+        if m.get("softcap"):
+            s = m["softcap"] * torch.tanh(s / m["softcap"])
         s = s.masked_fill(~see, float("-inf"))
         out[:, hd] = torch.softmax(s, dim=-1) @ v[:, g]
     out = out.reshape(n, -1) * torch.sigmoid(h @ W[p + "g"].T)
@@ -160,9 +164,10 @@ def delta(h: torch.Tensor, W: Dict[str, torch.Tensor], p: str, m: dict, eps: flo
 
 # ---------------------------------------------------------------------------------------------- feed-forward, model
 def dense_ff(h, W, p, mlp):
-    lim = mlp["limit"]
-    g = torch.clamp(h @ W[p + "gate"].T, max=lim)
-    u = torch.clamp(h @ W[p + "up"].T, -lim, lim)
+    lim = mlp.get("limit")
+    g, u = h @ W[p + "gate"].T, h @ W[p + "up"].T
+    if lim is not None:
+        g, u = torch.clamp(g, max=lim), torch.clamp(u, -lim, lim)
     return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ W[p + "down"].T
 
 
@@ -184,3 +189,15 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: List[int], laye
         if layers_out is not None:
             layers_out.append(x.clone())
     return norm_one_plus(x, W["final.norm"], eps) @ W["head"].T
+
+
+def greedy(cfg, weights, prompt: List[int], n_new: int):
+    """(tokens generated greedily, top-1 margin of every step)."""
+    toks, out, margins = list(prompt), [], []
+    for _ in range(n_new):
+        last = forward(cfg, weights, toks)[-1]
+        top = torch.topk(last, 2).values
+        out.append(int(torch.argmax(last)))
+        margins.append(float(top[0] - top[1]))
+        toks.append(out[-1])
+    return out, margins
