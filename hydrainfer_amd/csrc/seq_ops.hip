@@ -52,6 +52,57 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(typename A::storage* y
   }
 }
 
+// The same for up to MT taps, a thread keeping one channel's last inputs in registers over a tile of kConvTile tokens: every
+// input is read once instead of once per tap.  A tile may hold the ends and starts of several sequences: the history is
+// taken afresh (from the rows before, the slot, or zeros) at the tile's first token and at every portion's first token.
+constexpr int kConvTile = 16;
+
+template <typename A, int MT>
+__global__ __launch_bounds__(256) void causal_conv_tile_kernel(typename A::storage* y, int64_t y_stride, const typename A::storage* u,
+                                                               int64_t u_stride, const float* w, const float* bias, int act,
+                                                               const float* state, int64_t slot_stride, const int32_t* slots,
+                                                               const int32_t* tok_seq, const int32_t* q_cu, const int32_t* positions,
+                                                               int64_t T, int C, int taps) {
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int64_t tile0 = (int64_t)blockIdx.x * kConvTile;
+  const int64_t tile1 = tile0 + kConvTile < T ? tile0 + kConvTile : T;
+  const int keep = taps - 1;
+  float wt[MT], hist[MT];           // wt[j]: the weight of the input j tokens back; hist[j]: the input j + 1 tokens back
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    wt[j] = j < taps ? w[(int64_t)c * taps + (taps - 1 - j)] : 0.f;
+    hist[j] = 0.f;
+  }
+  const float b = bias ? bias[c] : 0.f;
+  for (int64_t t = tile0; t < tile1; ++t) {
+    const int seq = tok_seq[t];
+    const int64_t t0 = q_cu[seq];
+    if (t == tile0 || t == t0) {
+      const bool fresh = positions[t0] == 0;
+      const float* st = state + (int64_t)slots[seq] * slot_stride;
+#pragma unroll
+      for (int j = 0; j < MT - 1; ++j) {
+        const int64_t src = t - 1 - j;
+        float x = 0.f;
+        if (j < keep) {
+          if (src >= t0) x = A::to_float(u[src * u_stride + c]);
+          else if (!fresh) x = st[(int64_t)(keep - (int)(t0 - src)) * C + c];
+        }
+        hist[j] = x;
+      }
+    }
+    const float x = A::to_float(u[t * u_stride + c]);
+    float acc = b + wt[0] * x;
+#pragma unroll
+    for (int j = 0; j < MT - 1; ++j) acc += wt[j + 1] * hist[j];
+    y[t * y_stride + c] = A::from_float(act_apply(acc, act));
+#pragma unroll
+    for (int j = MT - 2; j > 0; --j) hist[j] = hist[j - 1];
+    hist[0] = x;
+  }
+}
+
 // the slot afterwards: the last taps - 1 inputs of (what the slot held, then the portion); one thread a channel, ascending
 template <typename A>
 __global__ __launch_bounds__(256) void causal_conv_state_kernel(const typename A::storage* u, int64_t u_stride, float* state,
@@ -79,12 +130,28 @@ template <typename A>
 __global__ __launch_bounds__(256) void token_shift_mix_kernel(typename A::storage* out, const typename A::storage* h, int64_t h_stride,
                                                               const float* mu, int n_mix, const float* state, int64_t slot_stride,
                                                               const int32_t* slots, const int32_t* tok_seq, const int32_t* q_cu,
-                                                              const int32_t* positions, int64_t T, int64_t W) {
+                                                              const int32_t* positions, int64_t T, int64_t W, int vec) {
   const int64_t t = blockIdx.x;
   const int seq = tok_seq[t];
   const int64_t t0 = q_cu[seq];
   const bool first = t == t0, fresh = positions[t0] == 0;
   const float* st = state + (int64_t)slots[seq] * slot_stride;
+  if (vec) {
+    for (int64_t c = 4 * (int64_t)threadIdx.x; c < W; c += 1024) {
+      const f32x4 x = Row4<A>::load(h + t * h_stride + c);
+      f32x4 prev = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (!first) prev = Row4<A>::load(h + (t - 1) * h_stride + c);
+      else if (!fresh) prev = *reinterpret_cast<const f32x4*>(st + c);
+      for (int m = 0; m < n_mix; ++m) {
+        const f32x4 w = *reinterpret_cast<const f32x4*>(mu + (int64_t)m * W + c);
+        f32x4 o;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) o[k] = x[k] + (prev[k] - x[k]) * w[k];
+        Row4<A>::store(out + ((int64_t)m * T + t) * W + c, o);
+      }
+    }
+    return;
+  }
   for (int64_t c = threadIdx.x; c < W; c += 256) {
     const float x = A::to_float(h[t * h_stride + c]);
     const float prev = first ? (fresh ? 0.f : st[c]) : A::to_float(h[(t - 1) * h_stride + c]);
@@ -190,56 +257,63 @@ __global__ __launch_bounds__(256) void unit_norm_kernel(float* out, const typena
 }
 
 // ------------------------------------------------------------------------------------------------ head norm + rotation + cache
-// one wave per (token, head): heads 0 .. q_heads - 1 are queries, the rest keys.  LDS: a head's normed channels per wave.
+// one workgroup per token: the token's cos and sin of every pair go once into LDS, then the four waves take the heads in
+// turn (heads 0 .. q_heads - 1 are queries, the rest keys).  LDS: [cos | sin] of the pairs, then a head's normed channels per wave.
 template <typename A>
 __global__ __launch_bounds__(256) void head_norm_rope_cache_kernel(hxm_head_rope_args a) {
   extern __shared__ float lds[];
   typedef typename A::storage T;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int NH = a.q_heads + a.kv_heads, D = a.dim, R = a.rot_dims, half = R >> 1;
-  const int64_t item = (int64_t)blockIdx.x * 4 + wave;
-  if (item >= a.n_tokens * NH) return;
-  const int64_t t = item / NH;
-  const int h = (int)(item - t * NH);
-  const bool is_q = h < a.q_heads;
-  const int g = is_q ? h : h - a.q_heads;
-  const T* x = is_q ? (const T*)a.q + t * a.q_stride + (int64_t)g * D : (const T*)a.k + t * a.k_stride + (int64_t)g * D;
-  const float* w = is_q ? a.q_w : a.k_w;
-  float* nb = lds + wave * D;
-  T* vrow = nullptr;
-  T* orow;
-  if (is_q) {
-    orow = (T*)a.q_out + (t * a.q_heads + g) * D;
-  } else {
-    const int64_t slot = a.slot_ids[t];
-    orow = (T*)a.key_cache + slot * a.cache_row_stride + (int64_t)g * a.head_stride;
-    vrow = (T*)a.value_cache + slot * a.cache_row_stride + (int64_t)g * a.head_stride;
-  }
-  float ss = 0.f;
-  for (int d = lane; d < D; d += 64) {
-    const T raw = x[d];
-    const float v = A::to_float(raw);
-    if (vrow) vrow[d] = raw;
-    ss += v * v;
-  }
-  ss = wave_sum(ss);
-  const float inv = 1.0f / sqrtf(ss / (float)D + a.eps);
-  for (int d = lane; d < D; d += 64) nb[d] = A::to_float(x[d]) * inv * w[d];
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const int64_t t = blockIdx.x;
+  float* cs = lds;
+  float* sn = lds + half;
+  float* nb = lds + 2 * half + wave * D;
   const float p = (float)a.positions[t];
-  for (int d = lane; d < D; d += 64) {
-    float o = nb[d];
-    if (d < R) {
-      const int i = d < half ? d : d - half;
-      float sn, cs;
-      sincosf(p * a.inv_freq[i], &sn, &cs);
-      sn *= a.cos_sin_scale;
-      cs *= a.cos_sin_scale;
-      o = d < half ? nb[d] * cs - nb[d + half] * sn : nb[d] * cs + nb[d - half] * sn;
+  for (int i = threadIdx.x; i < half; i += 256) {
+    float s_, c_;
+    sincosf(p * a.inv_freq[i], &s_, &c_);
+    cs[i] = c_ * a.cos_sin_scale;
+    sn[i] = s_ * a.cos_sin_scale;
+  }
+  __syncthreads();
+  const int64_t slot = a.kv_heads ? a.slot_ids[t] : 0;
+  for (int h = wave; h < NH; h += 4) {
+    const bool is_q = h < a.q_heads;
+    const int g = is_q ? h : h - a.q_heads;
+    const T* x = is_q ? (const T*)a.q + t * a.q_stride + (int64_t)g * D : (const T*)a.k + t * a.k_stride + (int64_t)g * D;
+    const float* w = is_q ? a.q_w : a.k_w;
+    T* vrow = nullptr;
+    T* orow;
+    if (is_q) {
+      orow = (T*)a.q_out + (t * a.q_heads + g) * D;
+    } else {
+      orow = (T*)a.key_cache + slot * a.cache_row_stride + (int64_t)g * a.head_stride;
+      vrow = (T*)a.value_cache + slot * a.cache_row_stride + (int64_t)g * a.head_stride;
     }
-    orow[d] = A::from_float(o);
+    float ss = 0.f;
+    for (int d = lane; d < D; d += 64) {
+      const T raw = x[d];
+      const float v = A::to_float(raw);
+      if (vrow) vrow[d] = raw;
+      nb[d] = v;
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)D + a.eps);
+    for (int d = lane; d < D; d += 64) nb[d] = nb[d] * inv * w[d];      // (a lane rewrites the channels it wrote)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    for (int d = lane; d < D; d += 64) {
+      float o = nb[d];
+      if (d < half) o = nb[d] * cs[d] - nb[d + half] * sn[d];
+      else if (d < R) o = nb[d] * cs[d - half] + nb[d - half] * sn[d - half];
+      orow[d] = A::from_float(o);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();                                    // the next head's channels overwrite nb
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
 }
 
@@ -252,9 +326,26 @@ __device__ __forceinline__ float gn_value(const hxm_group_norm_args& a, int64_t 
   return v;
 }
 
-// one wave per (row, group): the group's sum of squares, then the elements once more
 template <typename A, typename X>
-__global__ __launch_bounds__(256) void gated_group_norm_kernel(hxm_group_norm_args a) {
+__device__ __forceinline__ f32x4 gn_value4(const hxm_group_norm_args& a, int64_t r, int64_t c) {
+  f32x4 v = Row4<X>::load((const typename X::storage*)a.x + r * a.x_stride + c);
+  if (a.skip) {
+    const f32x4 sk = Row4<A>::load((const typename A::storage*)a.skip + r * a.skip_stride + c);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] += a.skip_w[(uint32_t)(c + k) / (uint32_t)a.skip_group] * sk[k];
+  }
+  if (a.gate && a.gate_first) {
+    const f32x4 g = Row4<A>::load((const typename A::storage*)a.gate + r * a.gate_stride + c);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] *= act_apply(g[k], a.gate_act);
+  }
+  return v;
+}
+
+// one wave per (row, group): the group's sum of squares, then the elements once more (vec: four elements a lane, the first
+// 1024 of a group kept in registers between the two passes)
+template <typename A, typename X>
+__global__ __launch_bounds__(256) void gated_group_norm_kernel(hxm_group_norm_args a, int vec) {
   typedef typename A::storage T;
   const int lane = threadIdx.x & 63;
   const int64_t gs = a.group > 0 ? a.group : (a.n < 1024 ? a.n : 1024);        // no norm: the groups only deal the work
@@ -263,6 +354,46 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(hxm_group_norm_ar
   if (item >= a.rows * n_groups) return;
   const int64_t r = item / n_groups, c0 = (item - r * n_groups) * gs;
   const int64_t c1 = c0 + gs < a.n ? c0 + gs : a.n;
+  T* o = (T*)a.out + r * a.out_stride;
+  if (vec) {
+    f32x4 keep[4];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int64_t c = c0 + 4 * (lane + 64 * i);
+      if (c < c1) {
+        keep[i] = gn_value4<A, X>(a, r, c);
+        ss += (keep[i][0] * keep[i][0] + keep[i][1] * keep[i][1]) + (keep[i][2] * keep[i][2] + keep[i][3] * keep[i][3]);
+      }
+    }
+    if (a.group > 0)
+      for (int64_t c = c0 + 4 * (lane + 256); c < c1; c += 256) {
+        const f32x4 v = gn_value4<A, X>(a, r, c);
+        ss += (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+      }
+    float inv = 1.f;
+    if (a.group > 0) inv = 1.0f / sqrtf(wave_sum(ss) / (float)gs + a.eps);
+    auto finish = [&](f32x4 v, int64_t c) {
+      f32x4 g = f32x4{1.f, 1.f, 1.f, 1.f};
+      if (a.gate && !a.gate_first) g = Row4<A>::load((const T*)a.gate + r * a.gate_stride + c);
+      const uint32_t cw = a.w ? (uint32_t)c % (uint32_t)a.w_len : 0;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        float x = v[k] * inv;
+        if (a.w) x *= a.w[cw + k < (uint32_t)a.w_len ? cw + k : cw + k - (uint32_t)a.w_len];
+        if (a.gate && !a.gate_first) x *= act_apply(g[k], a.gate_act);
+        v[k] = x * a.scale;
+      }
+      Row4<A>::store(o + c, v);
+    };
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int64_t c = c0 + 4 * (lane + 64 * i);
+      if (c < c1) finish(keep[i], c);
+    }
+    for (int64_t c = c0 + 4 * (lane + 256); c < c1; c += 256) finish(gn_value4<A, X>(a, r, c), c);
+    return;
+  }
   float inv = 1.f;
   if (a.group > 0) {
     float ss = 0.f;
@@ -273,7 +404,6 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(hxm_group_norm_ar
     ss = wave_sum(ss);
     inv = 1.0f / sqrtf(ss / (float)gs + a.eps);
   }
-  T* o = (T*)a.out + r * a.out_stride;
   for (int64_t c = c0 + lane; c < c1; c += 64) {
     float v = gn_value<A, X>(a, r, c) * inv;
     if (a.w) v *= a.w[c % a.w_len];
@@ -307,11 +437,24 @@ extern "C" int hxm_causal_conv(void* y, int64_t y_stride, const void* u, int64_t
   hipStream_t s = (hipStream_t)stream;
   const unsigned cb = (unsigned)((channels + 255) / 256);
   const dim3 grid((unsigned)n_tokens, cb < 64 ? cb : 64), sgrid((unsigned)n_seq, cb < 64 ? cb : 64), block(256);
-  HXM_BY_DTYPE(dtype,
-               (causal_conv_kernel<F32><<<grid, block, 0, s>>>((float*)y, y_stride, (const float*)u, u_stride, w, bias, act, state, slot_stride,
-                                                               slots, tok_seq, q_cu, positions, channels, taps)),
-               (causal_conv_kernel<BF16><<<grid, block, 0, s>>>((u16*)y, y_stride, (const u16*)u, u_stride, w, bias, act, state, slot_stride,
-                                                                slots, tok_seq, q_cu, positions, channels, taps)))
+  const dim3 tgrid((unsigned)((n_tokens + kConvTile - 1) / kConvTile), cb);
+#define HXM_CONV_TILE(A, MT)                                                                                                              \
+  causal_conv_tile_kernel<A, MT><<<tgrid, block, 0, s>>>((A::storage*)y, y_stride, (const A::storage*)u, u_stride, w, bias, act, state,   \
+                                                         slot_stride, slots, tok_seq, q_cu, positions, n_tokens, channels, taps)
+  if (taps <= 8 && n_tokens >= kConvTile) {
+    if (taps <= 4) {
+      HXM_BY_DTYPE(dtype, (HXM_CONV_TILE(F32, 4)), (HXM_CONV_TILE(BF16, 4)))
+    } else {
+      HXM_BY_DTYPE(dtype, (HXM_CONV_TILE(F32, 8)), (HXM_CONV_TILE(BF16, 8)))
+    }
+  } else {
+    HXM_BY_DTYPE(dtype,
+                 (causal_conv_kernel<F32><<<grid, block, 0, s>>>((float*)y, y_stride, (const float*)u, u_stride, w, bias, act, state, slot_stride,
+                                                                 slots, tok_seq, q_cu, positions, channels, taps)),
+                 (causal_conv_kernel<BF16><<<grid, block, 0, s>>>((u16*)y, y_stride, (const u16*)u, u_stride, w, bias, act, state, slot_stride,
+                                                                  slots, tok_seq, q_cu, positions, channels, taps)))
+  }
+#undef HXM_CONV_TILE
   int rc = hxm::check_launch();
   if (rc != HX_OK || taps == 1) return rc;
   HXM_BY_DTYPE(dtype,
@@ -331,11 +474,14 @@ extern "C" int hxm_token_shift_mix(void* out, const void* h, int64_t h_stride, c
   if (h_stride < width) return HX_ERR_STRIDE;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)n_tokens), sgrid((unsigned)n_seq), block(256);
+  const uintptr_t es = dtype == HX_F32 ? 4 : 2;
+  const int vec = width % 4 == 0 && h_stride % 4 == 0 && slot_stride % 4 == 0 && (uintptr_t)h % (4 * es) == 0 && (uintptr_t)out % (4 * es) == 0 &&
+                  (uintptr_t)mu % 16 == 0 && (uintptr_t)state % 16 == 0;
   HXM_BY_DTYPE(dtype,
                (token_shift_mix_kernel<F32><<<grid, block, 0, s>>>((float*)out, (const float*)h, h_stride, mu, n_mix, state, slot_stride, slots,
-                                                                   tok_seq, q_cu, positions, n_tokens, width)),
+                                                                   tok_seq, q_cu, positions, n_tokens, width, vec)),
                (token_shift_mix_kernel<BF16><<<grid, block, 0, s>>>((u16*)out, (const u16*)h, h_stride, mu, n_mix, state, slot_stride, slots,
-                                                                    tok_seq, q_cu, positions, n_tokens, width)))
+                                                                    tok_seq, q_cu, positions, n_tokens, width, vec)))
   int rc = hxm::check_launch();
   if (rc != HX_OK) return rc;
   HXM_BY_DTYPE(dtype,
@@ -430,10 +576,10 @@ extern "C" int hxm_head_norm_rope_cache(const hxm_head_rope_args* args, void* st
   if (a.kv_heads && (!a.k || !a.k_w || !a.slot_ids || !a.key_cache || !a.value_cache)) return HX_ERR_NULL;
   if ((a.q_heads && a.q_stride < (int64_t)a.q_heads * a.dim) || (a.kv_heads && a.k_stride < (int64_t)a.kv_heads * a.dim)) return HX_ERR_STRIDE;
   if (a.kv_heads && (a.head_stride < a.dim || a.cache_row_stride < a.head_stride * a.kv_heads)) return HX_ERR_STRIDE;
-  const size_t lds = 4 * (size_t)a.dim * sizeof(float);
+  const size_t lds = (4 * (size_t)a.dim + (size_t)a.rot_dims) * sizeof(float);
   if (lds > 64 * 1024) return HX_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
-  const dim3 grid((unsigned)((a.n_tokens * (a.q_heads + a.kv_heads) + 3) / 4)), block(256);
+  const dim3 grid((unsigned)a.n_tokens), block(256);
   HXM_BY_DTYPE(a.dtype, (head_norm_rope_cache_kernel<F32><<<grid, block, lds, s>>>(a)),
                (head_norm_rope_cache_kernel<BF16><<<grid, block, lds, s>>>(a)))
   return hxm::check_launch();
@@ -442,7 +588,7 @@ extern "C" int hxm_head_norm_rope_cache(const hxm_head_rope_args* args, void* st
 extern "C" int hxm_gated_group_norm(const hxm_group_norm_args* args, void* stream) {
   if (!args) return HX_ERR_NULL;
   const hxm_group_norm_args& a = *args;
-  if (a.rows < 0 || a.n < 1 || a.group < 0 || (a.group > 0 && a.n % a.group) || (a.w && a.w_len < 1) || (a.skip && a.skip_group < 1))
+  if (a.rows < 0 || a.n < 1 || a.n > 0x7fffffff || a.group < 0 || (a.group > 0 && a.n % a.group) || (a.w && a.w_len < 1) || (a.skip && a.skip_group < 1))
     return HX_ERR_SHAPE;
   if (a.rows == 0) return HX_OK;
   if (!a.out || !a.x || (a.skip && !a.skip_w)) return HX_ERR_NULL;
@@ -452,11 +598,15 @@ extern "C" int hxm_gated_group_norm(const hxm_group_norm_args* args, void* strea
   const int64_t gs = a.group > 0 ? a.group : (a.n < 1024 ? a.n : 1024);
   const int64_t items = a.rows * ((a.n + gs - 1) / gs);
   const dim3 grid((unsigned)((items + 3) / 4)), block(256);
+  const uintptr_t es = a.dtype == HX_F32 ? 4 : 2, xs = a.x_dtype == HX_F32 ? 4 : 2;
+  auto by4 = [](const void* p, int64_t stride, uintptr_t e) { return ((uintptr_t)p % (4 * e)) == 0 && stride % 4 == 0; };
+  const int vec = gs % 4 == 0 && a.n % 4 == 0 && by4(a.x, a.x_stride, xs) && by4(a.out, a.out_stride, es) && by4(a.skip, a.skip_stride, es) &&
+                  by4(a.gate, a.gate_stride, es);
   if (a.dtype == HX_F32) {
-    gated_group_norm_kernel<F32, F32><<<grid, block, 0, s>>>(a);
+    gated_group_norm_kernel<F32, F32><<<grid, block, 0, s>>>(a, vec);
   } else if (a.dtype == HX_BF16) {
-    if (a.x_dtype == HX_F32) gated_group_norm_kernel<BF16, F32><<<grid, block, 0, s>>>(a);
-    else gated_group_norm_kernel<BF16, BF16><<<grid, block, 0, s>>>(a);
+    if (a.x_dtype == HX_F32) gated_group_norm_kernel<BF16, F32><<<grid, block, 0, s>>>(a, vec);
+    else gated_group_norm_kernel<BF16, BF16><<<grid, block, 0, s>>>(a, vec);
   } else {
     return HX_ERR_DTYPE;
   }

@@ -1,4 +1,4 @@
-"""`bench.py --design tetepel|kezolix`: prefill and decode throughput of a model design at sizes that resemble a real
+"""`bench.py --design tetepel|kezolix|fasanex`: prefill and decode throughput of a model design at sizes that resemble a real
 model's layers (random weights, a few layers), beside the Llama decoder at equal width / feed-forward / heads, and a table
 of the design's own kernels against the Llama path's like kernels, each as a fraction of its roofline (HBM bytes or MFMA
 flops, algorithmic counts).  Both models run their eager step (no captured graph / launch plan) on hand-built batches."""
@@ -43,6 +43,23 @@ def _kezolix(size: dict, dtype, dev):
     return KezolixForCausalLM.random_init(shape, dtype, dev, seed=0)
 
 
+def _fasanex(size: dict, dtype, dev):
+    """Four layers, a dense feed-forward each: state-space (heads of 64 channels over the model's width, a 128 x 64 state
+    each, 8 groups, 4 taps), attention beside time mixing (attention as wide as the Llama decoder's with a quarter of the
+    heads carrying keys, a window of 512, half of every head turning; time mixing heads of 64), the delta rule (128 x 128
+    states, half of the heads carrying queries and keys), and the parallel mixer once more."""
+    from hydrainfer_amd.model.fasanex import (AttentionSpec, FasanexForCausalLM, FasanexLayer, FasanexShape, FeedForwardSpec, MixerSpec,
+                                              RotarySpec, TimeMixSpec)
+    H, D, ff, W = size["heads"], size["dim"], size["ff"], size["width"]
+    ssm = MixerSpec("mamba2", heads=W // 64, vdim=64, conv=4, state=128, groups=8, norm_groups=1)
+    par = MixerSpec("parallel", left=AttentionSpec(H, H // 4, D, D, 3, 1.0 / math.sqrt(D), 30.0, 512, RotarySpec(D // 2, 10000.0, 8.0, 4096.0, 32.0, 1.0)),
+                    right=TimeMixSpec(H, 64, 64), left_scale=1.0, right_scale=1.0)
+    dl = MixerSpec("delta", heads=H, vdim=D, conv=4, dim=D, kv_heads=H // 2)
+    layers = [FasanexLayer(m, FeedForwardSpec(ff, 7.0)) for m in (ssm, par, dl, par)][:size["layers"]]
+    shape = FasanexShape(VOCAB, W, layers, norm_eps=1e-5, embedding_scale=1.0)
+    return FasanexForCausalLM.random_init(shape, dtype, dev, seed=0)
+
+
 def _llama(size: dict, dtype, dev):
     from hydrainfer_amd.model.llama import LlamaForCausalLM, LlamaShape
     shape = LlamaShape(size["width"], size["ff"], size["layers"], size["heads"], size["heads"], size["dim"], VOCAB)
@@ -77,6 +94,10 @@ def _batch(model, n_seqs: int, q_len: int, kv_len: int, dtype, dev):
                                               torch.arange(n_seqs, dtype=torch.int32, device=dev).repeat_interleave(q_len))
     ids = torch.randint(0, VOCAB, (n_seqs * q_len,), device=dev, dtype=torch.int32)
     return ids, pos, params
+
+
+# the models a design's throughput is set beside: the closest existing one first
+BESIDE = {"fasanex": ("kezolix", "llama")}
 
 
 def _time_eager(fn: Callable, dev, reps: int = 5, warm: int = 2) -> float:
@@ -126,7 +147,9 @@ def _row(name, us, nbytes=None, flops=None):
 def throughput(size_name: str, dtype, dev, prefill=(4, 1024), decode=(32, 1024), design: str = "tetepel") -> dict:
     size = SIZES[size_name]
     out = {}
-    for name, make in ((design, {"tetepel": _tetepel, "kezolix": _kezolix}[design]), ("llama", _llama)):
+    makers = {"tetepel": _tetepel, "kezolix": _kezolix, "fasanex": _fasanex, "llama": _llama}
+    beside = BESIDE.get(design, ("llama",))
+    for name, make in [(n, makers[n]) for n in (design,) + beside]:
         model = make(size, dtype, dev)
         if name == "llama":
             model.prepare_decode(max_rows=decode[0])
@@ -368,11 +391,154 @@ def kezolix_kernel_table(size_name: str, dtype, dev, T: int = 4096, n_seqs: int 
     return rows
 
 
+def fasanex_kernel_table(size_name: str, dtype, dev, T: int = 4096, n_seqs: int = 4, B: int = 32, ctx: int = 2048) -> dict:
+    """Every kernel of the Fasanex design at a prefill batch of T tokens (n_seqs portions) — attention and the scans also at
+    a decode batch of B sequences — beside the like kernels of the closest design (Kezolix: recurrent / attention hybrid)
+    and of the Llama path at the same sizes."""
+    from hydrainfer_amd._C.kernel import biased_attn as ba, depth_ops as do, seq_mix as sm
+    from hydrainfer_amd._C.kernel.recurrence import gated_recurrence
+    from hydrainfer_amd._C.kernel.stream_ops import SequenceState
+    from hydrainfer_amd.model.fasanex import RotarySpec
+    sz = SIZES[size_name]
+    W, ff, H, D = sz["width"], sz["ff"], sz["heads"], sz["dim"]
+    G, window = H // 4, 512
+    e = 2
+    rnd = lambda *s: torch.randn(s, device=dev).to(dtype)
+    f32 = lambda *s: torch.randn(s, device=dev)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev) if not torch.is_tensor(v) else v.to(torch.int32).to(dev)
+    rows: Dict[str, List[dict]] = {"fasanex": [], "kezolix": [], "llama": []}
+    add = lambda *a, **k: rows["fasanex"].append(_row(*a, **k))
+    kez = lambda *a, **k: rows["kezolix"].append(_row(*a, **k))
+    q_len = T // n_seqs
+    q_cu = i32(list(range(0, T + 1, q_len)))
+    pos = torch.arange(q_len, dtype=torch.int32, device=dev).repeat(n_seqs)
+    tok_seq = torch.arange(n_seqs, dtype=torch.int32, device=dev).repeat_interleave(q_len)
+    posd, qcud, seq_ids = i32([ctx - 1] * B), i32(list(range(B + 1))), i32(list(range(B)))
+    # residual + norms: the kernel both designs share
+    x, y, w1, w2 = f32(T, W), rnd(T, W), f32(W), f32(W)
+    us = _time_graph(lambda: do.depth_norm(x, dtype, 1e-5, y=y, post_w=w1, x_out=x, next_w=w2, rms=True), dev)
+    add("depth_norm (RMS norm of y into the residual + next norm)", us, T * W * (8 + 2 * e))
+    kez("depth_norm, mid-layer (the same kernel, layer norms)", _time_graph(lambda: do.depth_norm(x, dtype, 1e-5, y=y, post_w=w1, mult=0.5, x_out=x, next_w=w2), dev),
+        T * W * (8 + 2 * e))
+    gu, coef = rnd(T, 2 * ff), f32(4)
+    us = _time_graph(lambda: sm.clamped_glu(gu[:, :ff], gu[:, ff:], 7.0), dev)
+    add("clamped_glu", us, 3 * T * ff * e)
+    kez("poly_norm", _time_graph(lambda: do.poly_norm(gu[:, :ff], coef, 1e-5), dev), 2 * T * ff * e)
+    # state pieces of one slot: [conv tail | shift | S]
+    n_slots = max(n_seqs, B)
+    inner, gn, N, P = W, 8 * 128, 128, 64
+    C = inner + 2 * gn
+    state = torch.zeros((n_slots, 1, 3 * C + W + H * D * D), device=dev)
+    seq = SequenceState(state, i32(list(range(n_seqs))), tok_seq)
+    seqd = SequenceState(state, seq_ids, seq_ids)
+    off_S = 3 * C + W
+    proj = rnd(T, 2 * inner + 2 * gn + inner // P)
+    cw, cb = f32(C, 4), f32(C)
+    us = _time_graph(lambda: sm.causal_conv(proj[:, inner:inner + C], cw, cb, "silu", seq, 0, q_cu, pos), dev)
+    add(f"causal_conv + bias + silu ({C} channels, 4 taps)", us, 2 * T * C * e)
+    hh, mu = rnd(T, W), torch.rand(5, W, device=dev)
+    us = _time_graph(lambda: sm.token_shift_mix(hh, mu, seq, 3 * C, q_cu, pos), dev)
+    add("token_shift_mix (five mixes)", us, 6 * T * W * e)
+    # attention side
+    nb, nbd = (q_len + 15) // 16, (ctx + 15) // 16
+    kc, vc = rnd(n_seqs * nb, 16, G, D), rnd(n_seqs * nb, 16, G, D)
+    table, cu_b = i32(torch.randperm(n_seqs * nb)), i32(list(range(0, n_seqs * nb + 1, nb)))
+    slots = i32([int(table[s * nb + p // 16]) * 16 + p % 16 for s in range(n_seqs) for p in range(q_len)])
+    qk, qw, kw = rnd(T, (H + G) * D), f32(D), f32(D)
+    freq, cs = RotarySpec(D // 2, 10000.0, 8.0, 4096.0, 32.0, 1.0).frequencies()
+    inv = torch.tensor(freq, device=dev, dtype=torch.float32)
+    us = _time_graph(lambda: sm.head_norm_rope_cache(qk[:, :H * D], qk[:, H * D:], qw, kw, 1e-5, H, G, D, inv, cs, pos, slots, kc, vc), dev)
+    add("head_norm_rope_cache (head norms + rotation + cache append)", us, T * (2 * H * D + 3 * G * D) * e)
+    qkv, qw2, kw2 = rnd(T, (H + 2 * G) * D), f32(H * D), f32(G * D)
+    kez("qk_norm_cache (two norms + cache append)", _time_graph(lambda: ba.qk_norm_cache(qkv, H * D, G * D, G * D, qw2, kw2, 1e-5, G, slots, kc, vc), dev),
+        T * (2 * H * D + 2 * G * D + 2 * G * D) * e)
+    q = rnd(T, H, D)
+    seen = n_seqs * sum(min(i + 1, window) for i in range(q_len))
+    us = _time_graph(lambda: ba.biased_attention(q, kc, vc, D, tok_seq, pos, q_cu, table, cu_b, 1 / math.sqrt(D), None, "window", window,
+                                                 max_q_len=q_len, max_kv_len=q_len, softcap=30.0), dev, launches=2)
+    add(f"biased_attention, prefill {n_seqs} x {q_len} (window {window}, soft cap, head_dim {D})", us, flops=4 * H * D * seen)
+    slopes = torch.tensor([2.0 ** (-8.0 * (h + 1) / H) for h in range(H)], device=dev)
+    seen_c = n_seqs * sum(i % window + 1 for i in range(q_len))
+    kez(f"biased_attention, prefill {n_seqs} x {q_len} (chunks of {window}, distance bias)",
+        _time_graph(lambda: ba.biased_attention(q, kc, vc, D, tok_seq, pos, q_cu, table, cu_b, 1 / math.sqrt(D), slopes, "chunk", window,
+                                                max_q_len=q_len, max_kv_len=q_len), dev, launches=2), flops=4 * H * D * seen_c)
+    kcd, vcd = rnd(B * nbd, 16, G, D), rnd(B * nbd, 16, G, D)
+    table_d, cu_bd = i32(torch.randperm(B * nbd)), i32(list(range(0, B * nbd + 1, nbd)))
+    qd = rnd(B, H, D)
+    us = _time_graph(lambda: ba.biased_attention(qd, kcd, vcd, D, seq_ids, posd, qcud, table_d, cu_bd, 1 / math.sqrt(D), None, "window", window,
+                                                 max_q_len=1, max_kv_len=ctx, softcap=30.0), dev)
+    add(f"biased_attention, decode {B} x {window} keys of the window (soft cap)", us, 2 * B * window * G * D * e + 2 * B * H * D * e)
+    pos_chunk_end = i32([window * (ctx // window) - 1] * B)
+    kez(f"biased_attention, decode {B} x {window} keys of its chunk",
+        _time_graph(lambda: ba.biased_attention(qd, kcd, vcd, D, seq_ids, pos_chunk_end, qcud, table_d, cu_bd,
+                                                1 / math.sqrt(D), slopes, "chunk", window, max_q_len=1, max_kv_len=ctx), dev),
+        2 * B * window * G * D * e + 2 * B * H * D * e)
+    og, gate = rnd(T, H * D), rnd(T, H * D)
+    both = rnd(T, H * D + 64)
+    us = _time_graph(lambda: sm.gated_group_norm(og, dtype, gate=gate, gate_act="sigmoid", scale=0.8, out=both[:, :H * D]), dev)
+    add("gated_group_norm: sigmoid gate on the attention's result", us, 3 * T * H * D * e)
+    # the scans, each at a state of H x 128 x 128 floats a sequence (the state-space form: W / 64 heads of 128 x 64)
+    Hs = inner // P
+    xbc, dtr = rnd(T, C), rnd(T, Hs)
+    rate, bias = f32(Hs) * 0.3, f32(Hs)
+    us = _time_graph(lambda: sm.head_gates(dtr, rate, bias, want_step=True), dev)
+    add("head_gates (decay and step size of every head)", us, T * Hs * (e + 8))
+    decay, step, _ = sm.head_gates(dtr, rate, bias, want_step=True)
+    flops_state = lambda n_tok, heads, k, v, per: per * n_tok * heads * k * v
+    us = _time_graph(lambda: sm.state_scan("decay", xbc[:, inner + gn:], xbc[:, inner:inner + gn], xbc[:, :inner], decay, seq, off_S, q_cu, pos,
+                                           Hs, 8, N, P, vscale=step), dev, launches=2)
+    add(f"state_scan decay form, prefill {n_seqs} x {q_len} ({Hs} heads, state {N} x {P})", us, flops=flops_state(T, Hs, N, P, 5))
+    us = _time_graph(lambda: sm.state_scan("decay", xbc[:B, inner + gn:], xbc[:B, inner:inner + gn], xbc[:B, :inner], decay[:B].contiguous(), seqd,
+                                           off_S, qcud, posd, Hs, 8, N, P, vscale=step[:B].contiguous()), dev)
+    add(f"state_scan decay form, decode {B} sequences (state read and written)", us, 2 * B * Hs * N * P * 4)
+    Hr, Dr = H, 64
+    rkv, dch, bonus = rnd(3, T, Hr * Dr), torch.rand(T, Hr * Dr, device=dev) * 0.5 + 0.5, f32(Hr * Dr)
+    us = _time_graph(lambda: sm.decay_exp(rkv[0], bonus), dev)
+    add("decay_exp (a decay per key channel)", us, T * Hr * Dr * (e + 4))
+    us = _time_graph(lambda: sm.state_scan("bonus", rkv[0], rkv[1], rkv[2], dch, seq, off_S, q_cu, pos, Hr, Hr, Dr, Dr, bonus=bonus), dev, launches=2)
+    add(f"state_scan bonus form, prefill {n_seqs} x {q_len} ({Hr} heads, state {Dr} x {Dr})", us, flops=flops_state(T, Hr, Dr, Dr, 7))
+    us = _time_graph(lambda: sm.state_scan("bonus", rkv[0, :B], rkv[1, :B], rkv[2, :B], dch[:B].contiguous(), seqd, off_S, qcud, posd, Hr, Hr, Dr, Dr,
+                                           bonus=bonus), dev)
+    add(f"state_scan bonus form, decode {B} sequences", us, 2 * B * Hr * Dr * Dr * 4)
+    Gd = H // 2
+    cqkv = rnd(T, 2 * Gd * D + H * D)
+    us = _time_graph(lambda: sm.unit_norm(cqkv[:, :Gd * D], Gd, D, 1e-6, D ** -0.5), dev)
+    add("unit_norm (queries or keys of the delta rule)", us, T * Gd * D * (e + 4))
+    qn, kn = sm.unit_norm(cqkv[:, :Gd * D], Gd, D, 1e-6, D ** -0.5), sm.unit_norm(cqkv[:, Gd * D:2 * Gd * D], Gd, D, 1e-6)
+    ab = rnd(T, 2 * H)
+    dec_d, _, beta = sm.head_gates(ab[:, H:], f32(H) * 0.3, f32(H), b=ab[:, :H])
+    us = _time_graph(lambda: sm.state_scan("delta", qn, kn, cqkv[:, 2 * Gd * D:], dec_d, seq, off_S, q_cu, pos, H, Gd, D, D, beta=beta), dev, launches=2)
+    add(f"state_scan delta form, prefill {n_seqs} x {q_len} ({H} heads, state {D} x {D})", us, flops=flops_state(T, H, D, D, 8))
+    us = _time_graph(lambda: sm.state_scan("delta", qn[:B], kn[:B], cqkv[:B, 2 * Gd * D:], dec_d[:B].contiguous(), seqd, off_S, qcud, posd, H, Gd, D, D,
+                                           beta=beta[:B].contiguous()), dev)
+    add(f"state_scan delta form, decode {B} sequences (state read and written)", us, 2 * B * H * D * D * 4)
+    o32, nw = f32(T, H * D), f32(D)
+    us = _time_graph(lambda: sm.gated_group_norm(o32, dtype, group=D, eps=1e-5, w=nw, gate=gate, gate_act="silu"), dev)
+    add("gated_group_norm: head norm + weight + silu gate after a scan", us, T * H * D * (4 + 2 * e))
+    # the closest design's recurrence at the same state size
+    pr = rnd(T, 3 * H * D)
+    fb, low, nw2 = f32(H * D), torch.rand(H * D, device=dev), f32(D)
+    st2 = torch.zeros((n_slots, 1, H * D * D), device=dev)
+    sq2, sq2d = SequenceState(st2, i32(list(range(n_seqs))), tok_seq), SequenceState(st2, seq_ids, seq_ids)
+    kez(f"gated_recurrence (scan + head norm), prefill {n_seqs} x {q_len} ({H} heads, state {D} x {D})",
+        _time_graph(lambda: gated_recurrence(pr[:, :H * D], pr[:, H * D:2 * H * D], pr[:, 2 * H * D:], fb, low, nw2, 1e-5, sq2, 0, q_cu, pos, H, D, D), dev,
+                    launches=2), flops=flops_state(T, H, D, D, 6))
+    kez(f"gated_recurrence, decode {B} sequences (state read and written)",
+        _time_graph(lambda: gated_recurrence(pr[:B, :H * D], pr[:B, H * D:2 * H * D], pr[:B, 2 * H * D:], fb, low, nw2, 1e-5, sq2d, 0, qcud, posd, H, D, D,
+                                             max_q_len=1), dev), 2 * B * H * D * D * 4)
+    rows["llama"] = _llama_rows(size_name, dtype, dev, T, n_seqs, B, ctx)
+    rows["workload"] = {"prefill_tokens": T, "portions": n_seqs, "decode_batch": B, "decode_keys": ctx, "size": sz,
+                        "timing": "hipGraph of 10 (long kernels: 2) launches, mean of 3 replays, HIP events",
+                        "roofline": f"HBM {HBM_PEAK_GBS} GB/s, MFMA {MFMA_PEAK_TFLOPS} TFLOP/s dense bf16; algorithmic bytes / flops "
+                                    "(the scans are float vector work: their flops are counted, not priced against the MFMA peak)"}
+    return rows
+
+
 def run(dtype, dev, sizes=("w2048", "w4096"), design: str = "tetepel") -> dict:
     from hydrainfer_amd import _lib
     _lib.lib(); _lib.mix_lib()
     res = {"throughput": {}, "kernels": {}}
-    table = {"tetepel": kernel_table, "kezolix": kezolix_kernel_table}[design]
+    table = {"tetepel": kernel_table, "kezolix": kezolix_kernel_table, "fasanex": fasanex_kernel_table}[design]
     for s in sizes:
         res["throughput"][s] = throughput(s, dtype, dev, design=design)
         res["kernels"][s] = table(s, dtype, dev)
