@@ -75,7 +75,13 @@ __global__ __launch_bounds__(256) void causal_conv_tile_kernel(typename A::stora
     hist[j] = 0.f;
   }
   const float b = bias ? bias[c] : 0.f;
-  for (int64_t t = tile0; t < tile1; ++t) {
+  float xs[kConvTile];              // the tile's inputs, all requested before the first is used
+#pragma unroll
+  for (int i = 0; i < kConvTile; ++i) xs[i] = tile0 + i < tile1 ? A::to_float(u[(tile0 + i) * u_stride + c]) : 0.f;
+#pragma unroll
+  for (int i = 0; i < kConvTile; ++i) {
+    const int64_t t = tile0 + i;
+    if (t >= tile1) break;
     const int seq = tok_seq[t];
     const int64_t t0 = q_cu[seq];
     if (t == tile0 || t == t0) {
@@ -92,7 +98,7 @@ __global__ __launch_bounds__(256) void causal_conv_tile_kernel(typename A::stora
         hist[j] = x;
       }
     }
-    const float x = A::to_float(u[t * u_stride + c]);
+    const float x = xs[i];
     float acc = b + wt[0] * x;
 #pragma unroll
     for (int j = 0; j < MT - 1; ++j) acc += wt[j + 1] * hist[j];
@@ -257,8 +263,9 @@ __global__ __launch_bounds__(256) void unit_norm_kernel(float* out, const typena
 }
 
 // ------------------------------------------------------------------------------------------------ head norm + rotation + cache
-// one workgroup per token: the token's cos and sin of every pair go once into LDS, then the four waves take the heads in
-// turn (heads 0 .. q_heads - 1 are queries, the rest keys).  LDS: [cos | sin] of the pairs, then a head's normed channels per wave.
+// one workgroup per token: the token's cos and sin of every pair and all its query and key heads go once into LDS (one
+// round trip to memory), then the four waves take the heads in turn (heads 0 .. q_heads - 1 are queries, the rest keys).
+// LDS: [cos | sin] of the pairs, then (q_heads + kv_heads) * dim floats.
 template <typename A>
 __global__ __launch_bounds__(256) void head_norm_rope_cache_kernel(hxm_head_rope_args a) {
   extern __shared__ float lds[];
@@ -268,7 +275,12 @@ __global__ __launch_bounds__(256) void head_norm_rope_cache_kernel(hxm_head_rope
   const int64_t t = blockIdx.x;
   float* cs = lds;
   float* sn = lds + half;
-  float* nb = lds + 2 * half + wave * D;
+  float* all = lds + 2 * half;
+  const int nq = a.q_heads * D, nk = a.kv_heads * D;
+  const T* qrow = (const T*)a.q + t * a.q_stride;
+  const T* krow = (const T*)a.k + t * a.k_stride;
+  for (int e = threadIdx.x; e < nq; e += 256) all[e] = A::to_float(qrow[e]);
+  for (int e = threadIdx.x; e < nk; e += 256) all[nq + e] = A::to_float(krow[e]);
   const float p = (float)a.positions[t];
   for (int i = threadIdx.x; i < half; i += 256) {
     float s_, c_;
@@ -278,10 +290,82 @@ __global__ __launch_bounds__(256) void head_norm_rope_cache_kernel(hxm_head_rope
   }
   __syncthreads();
   const int64_t slot = a.kv_heads ? a.slot_ids[t] : 0;
+  if (D % 2 == 0 && R % 4 == 0 && D <= 512 && (((uintptr_t)a.q_w | (uintptr_t)a.k_w) & 7) == 0) {
+    // two neighbouring channels a lane, the same ones for every head: their cos and sin stay in registers, the sum of
+    // squares is a DPP row sum and four lane reads, and a head costs three LDS accesses a lane
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    f32x2 c2[4], s2[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int d = 2 * (lane + 64 * i);
+      c2[i] = f32x2{1.f, 1.f};
+      s2[i] = f32x2{0.f, 0.f};
+      if (d < R) {
+        const int j = d < half ? d : d - half;
+        c2[i] = *reinterpret_cast<const f32x2*>(cs + j);
+        s2[i] = *reinterpret_cast<const f32x2*>(sn + j);
+        if (d < half) s2[i] = -s2[i];                 // the first half turns against its partner, the second with it
+      }
+    }
+    for (int h = wave; h < NH; h += 4) {
+      const bool is_q = h < a.q_heads;
+      const int g = is_q ? h : h - a.q_heads;
+      float* nb = all + (int64_t)h * D;
+      const float* w = is_q ? a.q_w : a.k_w;
+      T* orow = is_q ? (T*)a.q_out + (t * a.q_heads + g) * D : (T*)a.key_cache + slot * a.cache_row_stride + (int64_t)g * a.head_stride;
+      T* vrow = is_q ? nullptr : (T*)a.value_cache + slot * a.cache_row_stride + (int64_t)g * a.head_stride;
+      f32x2 x[4];
+      float ss = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int d = 2 * (lane + 64 * i);
+        x[i] = f32x2{0.f, 0.f};
+        if (d < D) {
+          x[i] = *reinterpret_cast<const f32x2*>(nb + d);
+          if (vrow) { vrow[d] = A::from_float(x[i][0]); vrow[d + 1] = A::from_float(x[i][1]); }
+          ss += x[i][0] * x[i][0] + x[i][1] * x[i][1];
+        }
+      }
+      ss = row16_sum(ss);
+      const float tot = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ss), 0)) +
+                        __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ss), 16)) +
+                        __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ss), 32)) +
+                        __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ss), 48));
+      const float inv = 1.0f / sqrtf(tot / (float)D + a.eps);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int d = 2 * (lane + 64 * i);
+        if (d < D) {
+          const f32x2 w2 = *reinterpret_cast<const f32x2*>(w + d);
+          x[i][0] *= inv * w2[0];
+          x[i][1] *= inv * w2[1];
+          if (d < R) *reinterpret_cast<f32x2*>(nb + d) = x[i];
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int d = 2 * (lane + 64 * i);
+        if (d < D) {
+          f32x2 o = x[i];
+          if (d < R) {
+            const f32x2 pr = *reinterpret_cast<const f32x2*>(nb + (d < half ? d + half : d - half));
+            o[0] = x[i][0] * c2[i][0] + pr[0] * s2[i][0];
+            o[1] = x[i][1] * c2[i][1] + pr[1] * s2[i][1];
+          }
+          orow[d] = A::from_float(o[0]);
+          orow[d + 1] = A::from_float(o[1]);
+        }
+      }
+    }
+    return;
+  }
   for (int h = wave; h < NH; h += 4) {
     const bool is_q = h < a.q_heads;
     const int g = is_q ? h : h - a.q_heads;
-    const T* x = is_q ? (const T*)a.q + t * a.q_stride + (int64_t)g * D : (const T*)a.k + t * a.k_stride + (int64_t)g * D;
+    float* nb = all + (int64_t)h * D;
     const float* w = is_q ? a.q_w : a.k_w;
     T* vrow = nullptr;
     T* orow;
@@ -293,15 +377,13 @@ __global__ __launch_bounds__(256) void head_norm_rope_cache_kernel(hxm_head_rope
     }
     float ss = 0.f;
     for (int d = lane; d < D; d += 64) {
-      const T raw = x[d];
-      const float v = A::to_float(raw);
-      if (vrow) vrow[d] = raw;
-      nb[d] = v;
+      const float v = nb[d];
+      if (vrow) vrow[d] = A::from_float(v);          // (exactly the element that came in)
       ss += v * v;
     }
     ss = wave_sum(ss);
     const float inv = 1.0f / sqrtf(ss / (float)D + a.eps);
-    for (int d = lane; d < D; d += 64) nb[d] = nb[d] * inv * w[d];      // (a lane rewrites the channels it wrote)
+    for (int d = lane; d < D; d += 64) nb[d] = nb[d] * inv * w[d];      // (a lane rewrites the channels it read)
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -311,9 +393,6 @@ __global__ __launch_bounds__(256) void head_norm_rope_cache_kernel(hxm_head_rope
       else if (d < R) o = nb[d] * cs[d - half] + nb[d - half] * sn[d - half];
       orow[d] = A::from_float(o);
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();                                    // the next head's channels overwrite nb
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
 }
 
@@ -410,6 +489,42 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(hxm_group_norm_ar
     if (a.gate && !a.gate_first) v *= act_apply(A::to_float(((const T*)a.gate)[r * a.gate_stride + c]), a.gate_act);
     o[c] = A::from_float(v * a.scale);
   }
+}
+
+// Groups of at most 128 elements, four elements a lane: LPG lanes a group, 64 / LPG groups a wave; everything a group needs
+// is requested before its sum is known.
+template <typename A, typename X>
+__global__ __launch_bounds__(256) void gated_group_norm_small_kernel(hxm_group_norm_args a, int lpg) {
+  typedef typename A::storage T;
+  const int lane = threadIdx.x & 63;
+  const int64_t gs = a.group > 0 ? a.group : (a.n < 128 ? a.n : 128);
+  const int64_t n_groups = (a.n + gs - 1) / gs;
+  const int64_t item = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * (64 / lpg) + lane / lpg;
+  const int64_t r = item / n_groups, c0 = (item - r * n_groups) * gs;
+  const int64_t c1 = c0 + gs < a.n ? c0 + gs : a.n;
+  const int64_t c = c0 + 4 * (lane % lpg);
+  const bool ok = item < a.rows * n_groups && c < c1;
+  f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f}, g = f32x4{1.f, 1.f, 1.f, 1.f};
+  if (ok) {
+    v = gn_value4<A, X>(a, r, c);
+    if (a.gate && !a.gate_first) g = Row4<A>::load((const T*)a.gate + r * a.gate_stride + c);
+  }
+  float inv = 1.f;
+  if (a.group > 0) {
+    float ss = (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+    for (int off = lpg >> 1; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    inv = 1.0f / sqrtf(ss / (float)gs + a.eps);
+  }
+  if (!ok) return;
+  const uint32_t cw = a.w ? (uint32_t)c % (uint32_t)a.w_len : 0;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    float x = v[k] * inv;
+    if (a.w) x *= a.w[cw + k < (uint32_t)a.w_len ? cw + k : cw + k - (uint32_t)a.w_len];
+    if (a.gate && !a.gate_first) x *= act_apply(g[k], a.gate_act);
+    v[k] = x * a.scale;
+  }
+  Row4<A>::store((T*)a.out + r * a.out_stride + c, v);
 }
 
 inline unsigned flat_blocks(int64_t total) {
@@ -576,7 +691,7 @@ extern "C" int hxm_head_norm_rope_cache(const hxm_head_rope_args* args, void* st
   if (a.kv_heads && (!a.k || !a.k_w || !a.slot_ids || !a.key_cache || !a.value_cache)) return HX_ERR_NULL;
   if ((a.q_heads && a.q_stride < (int64_t)a.q_heads * a.dim) || (a.kv_heads && a.k_stride < (int64_t)a.kv_heads * a.dim)) return HX_ERR_STRIDE;
   if (a.kv_heads && (a.head_stride < a.dim || a.cache_row_stride < a.head_stride * a.kv_heads)) return HX_ERR_STRIDE;
-  const size_t lds = (4 * (size_t)a.dim + (size_t)a.rot_dims) * sizeof(float);
+  const size_t lds = ((size_t)(a.q_heads + a.kv_heads) * a.dim + (size_t)a.rot_dims) * sizeof(float);
   if (lds > 64 * 1024) return HX_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)a.n_tokens), block(256);
@@ -602,6 +717,19 @@ extern "C" int hxm_gated_group_norm(const hxm_group_norm_args* args, void* strea
   auto by4 = [](const void* p, int64_t stride, uintptr_t e) { return ((uintptr_t)p % (4 * e)) == 0 && stride % 4 == 0; };
   const int vec = gs % 4 == 0 && a.n % 4 == 0 && by4(a.x, a.x_stride, xs) && by4(a.out, a.out_stride, es) && by4(a.skip, a.skip_stride, es) &&
                   by4(a.gate, a.gate_stride, es);
+  const int64_t small_gs = a.group > 0 ? a.group : (a.n < 128 ? a.n : 128);
+  if (vec && small_gs <= 128) {
+    int lpg = 1;
+    while (4 * lpg < small_gs) lpg <<= 1;
+    const int64_t small_items = a.rows * ((a.n + small_gs - 1) / small_gs);
+    const int64_t waves = (small_items + 64 / lpg - 1) / (64 / lpg);
+    const dim3 sgrid((unsigned)((waves + 3) / 4));
+    if (a.dtype == HX_F32) gated_group_norm_small_kernel<F32, F32><<<sgrid, block, 0, s>>>(a, lpg);
+    else if (a.dtype == HX_BF16 && a.x_dtype == HX_F32) gated_group_norm_small_kernel<BF16, F32><<<sgrid, block, 0, s>>>(a, lpg);
+    else if (a.dtype == HX_BF16) gated_group_norm_small_kernel<BF16, BF16><<<sgrid, block, 0, s>>>(a, lpg);
+    else return HX_ERR_DTYPE;
+    return hxm::check_launch();
+  }
   if (a.dtype == HX_F32) {
     gated_group_norm_kernel<F32, F32><<<grid, block, 0, s>>>(a, vec);
   } else if (a.dtype == HX_BF16) {

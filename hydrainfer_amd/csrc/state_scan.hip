@@ -164,7 +164,7 @@ __global__ __launch_bounds__(256) void state_scan_kernel(hxm_state_scan_args a) 
     const float* sc = vs + TC * COLS;
     const int n_tok = (int)(t_end - t0 < TC ? t_end - t0 : TC);
     if (col0 + wave * CPW < V) {          // (a wave whose columns all lie past vdim only helps to bring the chunks in)
-      for (int j = 0; j < n_tok; ++j) {
+      auto token = [&](int j) {
         float q[KR], k[KR], d[VEC ? KR : 1];
 #pragma unroll
         for (int r = 0; r < KR / 4; ++r) {
@@ -213,6 +213,12 @@ __global__ __launch_bounds__(256) void state_scan_kernel(hxm_state_scan_args a) 
         }
         o = parts_sum<PARTS>(o);
         if (part == 0 && col_ok) a.out[(t0 + j) * ((int64_t)a.heads * V) + (int64_t)head * V + col] = o;
+      };
+      if (n_tok == TC) {                  // a whole chunk: unrolled, so that the reads of the next tokens start early
+#pragma unroll 4
+        for (int j = 0; j < TC; ++j) token(j);
+      } else {
+        for (int j = 0; j < n_tok; ++j) token(j);
       }
     }
     if (more) store(lds + (cur ^ 1) * kImage);

@@ -319,7 +319,9 @@ def test_head_gates_decays_unit_norms_and_activations():
 
 @pytest.mark.parametrize("n,group,w_len,gate,first,skip", [(48, 8, 8, "silu", False, False), (48, 24, 48, "silu", True, True),
                                                           (35, 7, 35, "silu", False, False), (30, 0, 0, "sigmoid", False, False),
-                                                          (2048, 2048, 2048, "silu", True, True)])
+                                                          (2048, 2048, 2048, "silu", True, True), (64, 0, 0, "sigmoid", False, False),
+                                                          (1280, 0, 0, "silu", False, True), (512, 256, 256, "silu", False, False),
+                                                          (384, 128, 128, "silu", False, True)])
 def test_gate_and_group_norm(n, group, w_len, gate, first, skip):
     from hydrainfer_amd._C.kernel.seq_mix import gated_group_norm
     g = torch.Generator().manual_seed(n + group)
