@@ -3,6 +3,8 @@
 // holds the last token's input), the clamped gated feed-forward activation, per-head decays / step sizes / write
 // strengths of a recurrence, unit norms, per-head RMS norm + rotary positions + cache append, and the gate / group norm
 // that finishes a mixer.  Everything that is not a matrix product's operand is float.
+#include <type_traits>
+
 #include "hx_common.h"
 #include "mix_rows.h"
 #include "../../include/hydra_mix.h"
@@ -16,10 +18,19 @@ namespace {
 
 using namespace hx;
 
+// A sigmoid for results that are rounded to bfloat16 right away: the hardware's exponential and reciprocal (about one unit
+// in the last place of a float each) instead of the library's exact forms; float32 activations take the exact ones.
+template <typename A>
+__device__ __forceinline__ float sigmoid_of(float x) {
+  if constexpr (A::kDtype == HX_F32) return 1.f / (1.f + expf(-x));
+  else return __builtin_amdgcn_rcpf(1.f + __expf(-x));
+}
+
+template <typename A>
 __device__ __forceinline__ float act_apply(float x, int act) {
   switch (act) {
-    case HXM_ACT_SILU: return x / (1.f + expf(-x));
-    case HXM_ACT_SIGMOID: return 1.f / (1.f + expf(-x));
+    case HXM_ACT_SILU: return x * sigmoid_of<A>(x);
+    case HXM_ACT_SIGMOID: return sigmoid_of<A>(x);
     case HXM_ACT_TANH: return tanhf(x);
     default: return x;
   }
@@ -48,7 +59,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(typename A::storage* y
       else if (!fresh) x = st[(int64_t)((taps - 1) - (int)(t0 - src)) * C + c];
       acc += w[(int64_t)c * taps + j] * x;
     }
-    y[t * y_stride + c] = A::from_float(act_apply(acc, act));
+    y[t * y_stride + c] = A::from_float(act_apply<A>(acc, act));
   }
 }
 
@@ -57,55 +68,102 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(typename A::storage* y
 // taken afresh (from the rows before, the slot, or zeros) at the tile's first token and at every portion's first token.
 constexpr int kConvTile = 16;
 
-template <typename A, int MT>
+template <typename A, int NC> struct Chan;      // NC neighbouring channels of an activation row at once
+template <typename A> struct Chan<A, 1> {
+  static __device__ __forceinline__ void load(const typename A::storage* p, float (&v)[1]) { v[0] = A::to_float(p[0]); }
+  static __device__ __forceinline__ void store(typename A::storage* p, const float (&v)[1]) { p[0] = A::from_float(v[0]); }
+};
+template <> struct Chan<F32, 2> {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  static __device__ __forceinline__ void load(const float* p, float (&v)[2]) {
+    const f32x2 t = *reinterpret_cast<const f32x2*>(p);
+    v[0] = t[0]; v[1] = t[1];
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[2]) { *reinterpret_cast<f32x2*>(p) = f32x2{v[0], v[1]}; }
+};
+template <> struct Chan<BF16, 2> {
+  static __device__ __forceinline__ void load(const u16* p, float (&v)[2]) {
+    const uint32_t t = *reinterpret_cast<const uint32_t*>(p);
+    v[0] = __builtin_bit_cast(float, t << 16); v[1] = __builtin_bit_cast(float, t & 0xffff0000u);
+  }
+  static __device__ __forceinline__ void store(u16* p, const float (&v)[2]) {
+    *reinterpret_cast<uint32_t*>(p) = (uint32_t)BF16::from_float(v[0]) | ((uint32_t)BF16::from_float(v[1]) << 16);
+  }
+};
+
+template <typename A, int MT, int NC>
 __global__ __launch_bounds__(256) void causal_conv_tile_kernel(typename A::storage* y, int64_t y_stride, const typename A::storage* u,
                                                                int64_t u_stride, const float* w, const float* bias, int act,
                                                                const float* state, int64_t slot_stride, const int32_t* slots,
                                                                const int32_t* tok_seq, const int32_t* q_cu, const int32_t* positions,
                                                                int64_t T, int C, int taps) {
-  const int c = blockIdx.y * 256 + threadIdx.x;
+  const int c = NC * (blockIdx.y * 256 + threadIdx.x);
   if (c >= C) return;
   const int64_t tile0 = (int64_t)blockIdx.x * kConvTile;
   const int64_t tile1 = tile0 + kConvTile < T ? tile0 + kConvTile : T;
   const int keep = taps - 1;
-  float wt[MT], hist[MT];           // wt[j]: the weight of the input j tokens back; hist[j]: the input j + 1 tokens back
+  float wt[NC][MT], hist[NC][MT], b[NC];    // wt[.][j]: the weight of the input j tokens back; hist[.][j]: the input j + 1 tokens back
 #pragma unroll
-  for (int j = 0; j < MT; ++j) {
-    wt[j] = j < taps ? w[(int64_t)c * taps + (taps - 1 - j)] : 0.f;
-    hist[j] = 0.f;
+  for (int n = 0; n < NC; ++n) {
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      wt[n][j] = j < taps ? w[(int64_t)(c + n) * taps + (taps - 1 - j)] : 0.f;
+      hist[n][j] = 0.f;
+    }
+    b[n] = bias ? bias[c + n] : 0.f;
   }
-  const float b = bias ? bias[c] : 0.f;
-  float xs[kConvTile];              // the tile's inputs, all requested before the first is used
+  // the tile's sequence ids and inputs are requested at once, before anything waits for them: a portion starts where
+  // the id changes, and only there (and at the tile's first token) is the history taken afresh
+  int sid[kConvTile];
+  float xs[kConvTile][NC];
 #pragma unroll
-  for (int i = 0; i < kConvTile; ++i) xs[i] = tile0 + i < tile1 ? A::to_float(u[(tile0 + i) * u_stride + c]) : 0.f;
+  for (int i = 0; i < kConvTile; ++i) {
+    const int64_t t = tile0 + i < tile1 ? tile0 + i : tile1 - 1;
+    sid[i] = tok_seq[t];
+    Chan<A, NC>::load(u + t * u_stride + c, xs[i]);
+  }
 #pragma unroll
   for (int i = 0; i < kConvTile; ++i) {
     const int64_t t = tile0 + i;
-    if (t >= tile1) break;
-    const int seq = tok_seq[t];
-    const int64_t t0 = q_cu[seq];
-    if (t == tile0 || t == t0) {
+    if (t < tile1) {
+    if (i == 0 || sid[i] != sid[i > 0 ? i - 1 : 0]) {
+      const int seq = sid[i];
+      const int64_t t0 = q_cu[seq];
       const bool fresh = positions[t0] == 0;
       const float* st = state + (int64_t)slots[seq] * slot_stride;
 #pragma unroll
       for (int j = 0; j < MT - 1; ++j) {
         const int64_t src = t - 1 - j;
-        float x = 0.f;
+        float x[NC];
+#pragma unroll
+        for (int n = 0; n < NC; ++n) x[n] = 0.f;
         if (j < keep) {
-          if (src >= t0) x = A::to_float(u[src * u_stride + c]);
-          else if (!fresh) x = st[(int64_t)(keep - (int)(t0 - src)) * C + c];
+          if (src >= t0) {
+            Chan<A, NC>::load(u + src * u_stride + c, x);
+          } else if (!fresh) {
+#pragma unroll
+            for (int n = 0; n < NC; ++n) x[n] = st[(int64_t)(keep - (int)(t0 - src)) * C + c + n];
+          }
         }
-        hist[j] = x;
+#pragma unroll
+        for (int n = 0; n < NC; ++n) hist[n][j] = x[n];
       }
     }
-    const float x = xs[i];
-    float acc = b + wt[0] * x;
+    float x[NC], o[NC];
 #pragma unroll
-    for (int j = 0; j < MT - 1; ++j) acc += wt[j + 1] * hist[j];
-    y[t * y_stride + c] = A::from_float(act_apply(acc, act));
+    for (int n = 0; n < NC; ++n) x[n] = xs[i][n];
 #pragma unroll
-    for (int j = MT - 2; j > 0; --j) hist[j] = hist[j - 1];
-    hist[0] = x;
+    for (int n = 0; n < NC; ++n) {
+      float acc = b[n] + wt[n][0] * x[n];
+#pragma unroll
+      for (int j = 0; j < MT - 1; ++j) acc += wt[n][j + 1] * hist[n][j];
+      o[n] = act_apply<A>(acc, act);
+#pragma unroll
+      for (int j = MT - 2; j > 0; --j) hist[n][j] = hist[n][j - 1];
+      hist[n][0] = x[n];
+    }
+    Chan<A, NC>::store(y + t * y_stride + c, o);
+    }
   }
 }
 
@@ -190,7 +248,7 @@ __global__ __launch_bounds__(256) void clamped_glu_kernel(typename A::storage* y
       for (int k = 0; k < 4; ++k) {
         const float gg = limit > 0.f ? fminf(g[k], limit) : g[k];
         const float uu = limit > 0.f ? fminf(fmaxf(u[k], -limit), limit) : u[k];
-        o[k] = gg / (1.f + expf(-alpha * gg)) * (uu + up_shift);
+        o[k] = gg * sigmoid_of<A>(alpha * gg) * (uu + up_shift);
       }
       Row4<A>::store(y + r * y_stride + i, o);
     }
@@ -202,7 +260,7 @@ __global__ __launch_bounds__(256) void clamped_glu_kernel(typename A::storage* y
     const float g = A::to_float(gate[r * gate_stride + i]), u = A::to_float(up[r * up_stride + i]);
     const float gg = limit > 0.f ? fminf(g, limit) : g;
     const float uu = limit > 0.f ? fminf(fmaxf(u, -limit), limit) : u;
-    y[r * y_stride + i] = A::from_float(gg / (1.f + expf(-alpha * gg)) * (uu + up_shift));
+    y[r * y_stride + i] = A::from_float(gg * sigmoid_of<A>(alpha * gg) * (uu + up_shift));
   }
 }
 
@@ -212,7 +270,7 @@ __global__ __launch_bounds__(256) void unary_kernel(typename A::storage* out, in
   const int64_t total = rows * n;
   for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (int64_t)gridDim.x * 256) {
     const int64_t r = e / n, i = e - r * n;
-    out[r * out_stride + i] = A::from_float(act_apply(A::to_float(x[r * x_stride + i]), act));
+    out[r * out_stride + i] = A::from_float(act_apply<A>(A::to_float(x[r * x_stride + i]), act));
   }
 }
 
@@ -263,6 +321,20 @@ __global__ __launch_bounds__(256) void unit_norm_kernel(float* out, const typena
 }
 
 // ------------------------------------------------------------------------------------------------ head norm + rotation + cache
+// two neighbouring elements of an activation row in one store (p on a multiple of two elements)
+template <typename A> struct Pair;
+template <> struct Pair<F32> {
+  static __device__ __forceinline__ void store(float* p, float a, float b) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    *reinterpret_cast<f32x2*>(p) = f32x2{a, b};
+  }
+};
+template <> struct Pair<BF16> {
+  static __device__ __forceinline__ void store(u16* p, float a, float b) {
+    *reinterpret_cast<uint32_t*>(p) = (uint32_t)BF16::from_float(a) | ((uint32_t)BF16::from_float(b) << 16);
+  }
+};
+
 // one workgroup per token: the token's cos and sin of every pair and all its query and key heads go once into LDS (one
 // round trip to memory), then the four waves take the heads in turn (heads 0 .. q_heads - 1 are queries, the rest keys).
 // LDS: [cos | sin] of the pairs, then (q_heads + kv_heads) * dim floats.
@@ -279,8 +351,15 @@ __global__ __launch_bounds__(256) void head_norm_rope_cache_kernel(hxm_head_rope
   const int nq = a.q_heads * D, nk = a.kv_heads * D;
   const T* qrow = (const T*)a.q + t * a.q_stride;
   const T* krow = (const T*)a.k + t * a.k_stride;
-  for (int e = threadIdx.x; e < nq; e += 256) all[e] = A::to_float(qrow[e]);
-  for (int e = threadIdx.x; e < nk; e += 256) all[nq + e] = A::to_float(krow[e]);
+  const bool rows4 = nq % 4 == 0 && nk % 4 == 0 && R % 2 == 0 && a.q_stride % 4 == 0 && a.k_stride % 4 == 0 &&
+                     (((uintptr_t)a.q | (uintptr_t)a.k) % (4 * sizeof(T))) == 0;
+  if (rows4) {
+    for (int e = 4 * threadIdx.x; e < nq; e += 1024) *reinterpret_cast<f32x4*>(all + e) = Row4<A>::load(qrow + e);
+    for (int e = 4 * threadIdx.x; e < nk; e += 1024) *reinterpret_cast<f32x4*>(all + nq + e) = Row4<A>::load(krow + e);
+  } else {
+    for (int e = threadIdx.x; e < nq; e += 256) all[e] = A::to_float(qrow[e]);
+    for (int e = threadIdx.x; e < nk; e += 256) all[nq + e] = A::to_float(krow[e]);
+  }
   const float p = (float)a.positions[t];
   for (int i = threadIdx.x; i < half; i += 256) {
     float s_, c_;
@@ -290,7 +369,9 @@ __global__ __launch_bounds__(256) void head_norm_rope_cache_kernel(hxm_head_rope
   }
   __syncthreads();
   const int64_t slot = a.kv_heads ? a.slot_ids[t] : 0;
-  if (D % 2 == 0 && R % 4 == 0 && D <= 512 && (((uintptr_t)a.q_w | (uintptr_t)a.k_w) & 7) == 0) {
+  const uintptr_t pair_bytes = 2 * sizeof(T);
+  if (D % 2 == 0 && R % 4 == 0 && D <= 512 && (((uintptr_t)a.q_w | (uintptr_t)a.k_w) & 7) == 0 && ((a.cache_row_stride | a.head_stride) & 1) == 0 &&
+      (((uintptr_t)a.q_out | (uintptr_t)a.key_cache | (uintptr_t)a.value_cache) % pair_bytes) == 0) {
     // two neighbouring channels a lane, the same ones for every head: their cos and sin stay in registers, the sum of
     // squares is a DPP row sum and four lane reads, and a head costs three LDS accesses a lane
     typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -322,7 +403,7 @@ __global__ __launch_bounds__(256) void head_norm_rope_cache_kernel(hxm_head_rope
         x[i] = f32x2{0.f, 0.f};
         if (d < D) {
           x[i] = *reinterpret_cast<const f32x2*>(nb + d);
-          if (vrow) { vrow[d] = A::from_float(x[i][0]); vrow[d + 1] = A::from_float(x[i][1]); }
+          if (vrow) Pair<A>::store(vrow + d, x[i][0], x[i][1]);
           ss += x[i][0] * x[i][0] + x[i][1] * x[i][1];
         }
       }
@@ -355,8 +436,7 @@ __global__ __launch_bounds__(256) void head_norm_rope_cache_kernel(hxm_head_rope
             o[0] = x[i][0] * c2[i][0] + pr[0] * s2[i][0];
             o[1] = x[i][1] * c2[i][1] + pr[1] * s2[i][1];
           }
-          orow[d] = A::from_float(o[0]);
-          orow[d + 1] = A::from_float(o[1]);
+          Pair<A>::store(orow + d, o[0], o[1]);
         }
       }
     }
@@ -401,7 +481,7 @@ template <typename A, typename X>
 __device__ __forceinline__ float gn_value(const hxm_group_norm_args& a, int64_t r, int64_t c) {
   float v = X::to_float(((const typename X::storage*)a.x)[r * a.x_stride + c]);
   if (a.skip) v += a.skip_w[c / a.skip_group] * A::to_float(((const typename A::storage*)a.skip)[r * a.skip_stride + c]);
-  if (a.gate && a.gate_first) v *= act_apply(A::to_float(((const typename A::storage*)a.gate)[r * a.gate_stride + c]), a.gate_act);
+  if (a.gate && a.gate_first) v *= act_apply<A>(A::to_float(((const typename A::storage*)a.gate)[r * a.gate_stride + c]), a.gate_act);
   return v;
 }
 
@@ -416,7 +496,7 @@ __device__ __forceinline__ f32x4 gn_value4(const hxm_group_norm_args& a, int64_t
   if (a.gate && a.gate_first) {
     const f32x4 g = Row4<A>::load((const typename A::storage*)a.gate + r * a.gate_stride + c);
 #pragma unroll
-    for (int k = 0; k < 4; ++k) v[k] *= act_apply(g[k], a.gate_act);
+    for (int k = 0; k < 4; ++k) v[k] *= act_apply<A>(g[k], a.gate_act);
   }
   return v;
 }
@@ -460,7 +540,7 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(hxm_group_norm_ar
       for (int k = 0; k < 4; ++k) {
         float x = v[k] * inv;
         if (a.w) x *= a.w[cw + k < (uint32_t)a.w_len ? cw + k : cw + k - (uint32_t)a.w_len];
-        if (a.gate && !a.gate_first) x *= act_apply(g[k], a.gate_act);
+        if (a.gate && !a.gate_first) x *= act_apply<A>(g[k], a.gate_act);
         v[k] = x * a.scale;
       }
       Row4<A>::store(o + c, v);
@@ -486,7 +566,7 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(hxm_group_norm_ar
   for (int64_t c = c0 + lane; c < c1; c += 64) {
     float v = gn_value<A, X>(a, r, c) * inv;
     if (a.w) v *= a.w[c % a.w_len];
-    if (a.gate && !a.gate_first) v *= act_apply(A::to_float(((const T*)a.gate)[r * a.gate_stride + c]), a.gate_act);
+    if (a.gate && !a.gate_first) v *= act_apply<A>(A::to_float(((const T*)a.gate)[r * a.gate_stride + c]), a.gate_act);
     o[c] = A::from_float(v * a.scale);
   }
 }
@@ -521,7 +601,7 @@ __global__ __launch_bounds__(256) void gated_group_norm_small_kernel(hxm_group_n
   for (int k = 0; k < 4; ++k) {
     float x = v[k] * inv;
     if (a.w) x *= a.w[cw + k < (uint32_t)a.w_len ? cw + k : cw + k - (uint32_t)a.w_len];
-    if (a.gate && !a.gate_first) x *= act_apply(g[k], a.gate_act);
+    if (a.gate && !a.gate_first) x *= act_apply<A>(g[k], a.gate_act);
     v[k] = x * a.scale;
   }
   Row4<A>::store((T*)a.out + r * a.out_stride + c, v);
@@ -552,15 +632,27 @@ extern "C" int hxm_causal_conv(void* y, int64_t y_stride, const void* u, int64_t
   hipStream_t s = (hipStream_t)stream;
   const unsigned cb = (unsigned)((channels + 255) / 256);
   const dim3 grid((unsigned)n_tokens, cb < 64 ? cb : 64), sgrid((unsigned)n_seq, cb < 64 ? cb : 64), block(256);
-  const dim3 tgrid((unsigned)((n_tokens + kConvTile - 1) / kConvTile), cb);
-#define HXM_CONV_TILE(A, MT)                                                                                                              \
-  causal_conv_tile_kernel<A, MT><<<tgrid, block, 0, s>>>((A::storage*)y, y_stride, (const A::storage*)u, u_stride, w, bias, act, state,   \
-                                                         slot_stride, slots, tok_seq, q_cu, positions, n_tokens, channels, taps)
+  const uintptr_t pair = dtype == HX_F32 ? 8 : 4;
+  const bool two = channels % 2 == 0 && y_stride % 2 == 0 && u_stride % 2 == 0 && (uintptr_t)y % pair == 0 && (uintptr_t)u % pair == 0;
+  const dim3 tgrid((unsigned)((n_tokens + kConvTile - 1) / kConvTile), two ? (unsigned)((channels / 2 + 255) / 256) : cb);
+  auto tile = [&](auto tag, auto mt) {
+    typedef decltype(tag) A;
+    constexpr int MT = decltype(mt)::value;
+    typedef typename A::storage E;
+    if (two)
+      causal_conv_tile_kernel<A, MT, 2><<<tgrid, block, 0, s>>>((E*)y, y_stride, (const E*)u, u_stride, w, bias, act, state, slot_stride, slots,
+                                                                tok_seq, q_cu, positions, n_tokens, channels, taps);
+    else
+      causal_conv_tile_kernel<A, MT, 1><<<tgrid, block, 0, s>>>((E*)y, y_stride, (const E*)u, u_stride, w, bias, act, state, slot_stride, slots,
+                                                                tok_seq, q_cu, positions, n_tokens, channels, taps);
+  };
+  typedef std::integral_constant<int, 4> Taps4;
+  typedef std::integral_constant<int, 8> Taps8;
   if (taps <= 8 && n_tokens >= kConvTile) {
     if (taps <= 4) {
-      HXM_BY_DTYPE(dtype, (HXM_CONV_TILE(F32, 4)), (HXM_CONV_TILE(BF16, 4)))
+      HXM_BY_DTYPE(dtype, (tile(F32{}, Taps4{})), (tile(BF16{}, Taps4{})))
     } else {
-      HXM_BY_DTYPE(dtype, (HXM_CONV_TILE(F32, 8)), (HXM_CONV_TILE(BF16, 8)))
+      HXM_BY_DTYPE(dtype, (tile(F32{}, Taps8{})), (tile(BF16{}, Taps8{})))
     }
   } else {
     HXM_BY_DTYPE(dtype,
@@ -569,7 +661,6 @@ extern "C" int hxm_causal_conv(void* y, int64_t y_stride, const void* u, int64_t
                  (causal_conv_kernel<BF16><<<grid, block, 0, s>>>((u16*)y, y_stride, (const u16*)u, u_stride, w, bias, act, state, slot_stride,
                                                                   slots, tok_seq, q_cu, positions, channels, taps)))
   }
-#undef HXM_CONV_TILE
   int rc = hxm::check_launch();
   if (rc != HX_OK || taps == 1) return rc;
   HXM_BY_DTYPE(dtype,
