@@ -11,7 +11,8 @@
 // chunk's q, k (and per-channel decays) come once per workgroup as float into LDS, zero-padded to PARTS * KR channels, and
 // are read back 16 bytes at a time; the next chunk is on its way into registers while the current one is scanned (two LDS
 // images, one barrier a chunk), so the serial chain waits for no global load.  The state comes from the sequence's slot
-// (zeros for a portion that starts at position 0) and goes back.
+// (zeros for a portion that starts at position 0) and goes back.  KR x PARTS follows the key size (8 x 4 ... 16 x 16); a
+// launch of prompts with few workgroups takes more lanes a column, a batch of single tokens two columns a lane.
 #include "hx_common.h"
 #include "mix_rows.h"
 #include "../../include/hydra_mix.h"

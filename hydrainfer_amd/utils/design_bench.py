@@ -1,7 +1,8 @@
 """`bench.py --design tetepel|kezolix|fasanex`: prefill and decode throughput of a model design at sizes that resemble a real
-model's layers (random weights, a few layers), beside the Llama decoder at equal width / feed-forward / heads, and a table
-of the design's own kernels against the Llama path's like kernels, each as a fraction of its roofline (HBM bytes or MFMA
-flops, algorithmic counts).  Both models run their eager step (no captured graph / launch plan) on hand-built batches."""
+model's layers (random weights, a few layers), beside the Llama decoder at equal width / feed-forward / heads (Fasanex:
+also beside Kezolix, the closest design), and a table of the design's own kernels against the like kernels of the models
+beside it, each as a fraction of its roofline (HBM bytes or MFMA flops, algorithmic counts).  All models run their eager
+step (no captured graph / launch plan) on hand-built batches."""
 import math
 import time
 from typing import Callable, Dict, List

@@ -6,7 +6,11 @@
  * norms around every sublayer with the residual kept in a stack of levels (depth-weighted average), the PolyNorm and
  * squared-ReLU activations, a softmax router with a choice bias, grouped expert products over expert-major rows, a
  * gated linear recurrence with a matrix state per head (HGRN2), and grouped-query attention over a paged key/value
- * cache with a per-head linear distance bias and a causal, windowed or chunked mask.
+ * cache with a per-head linear distance bias, an optional soft cap on the scores and a causal, windowed or chunked mask;
+ * and, for mixers that keep per-sequence state beside the cache: short causal convolutions, token shift with several
+ * mixes, per-head RMS norm + rotary positions + cache append, decays / step sizes / write strengths of a recurrence, a scan
+ * over a matrix state per head in three forms (decayed sum, read-before-write with a bonus, delta rule), the gate / group
+ * norm that finishes a mixer, and a clamped gated feed-forward activation.
  *
  * Same conventions as hydra_hip.h: raw device pointers, sizes and strides in ELEMENTS, a hipStream_t passed as void*,
  * asynchronous launches, no allocation, 0 or a negative hx_status (hydra_hip.h) as the result.  `dtype` is the hx_dtype
