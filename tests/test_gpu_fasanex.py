@@ -197,7 +197,7 @@ def _through_portions(fn, inputs, n_a, n_b, floats):
 
 # ------------------------------------------------------------------------------------------------ mechanisms alone
 @pytest.mark.parametrize("C,taps,bias,act", [(38, 4, True, "silu"), (64, 3, False, None), (7, 1, False, "silu"), (130, 5, True, None),
-                                             (16, 2, False, "silu")])
+                                             (16, 2, False, "silu"), (20, 9, True, "silu"), (600, 8, False, None)])
 def test_short_convolution_through_portions_and_slots(C, taps, bias, act):
     from hydrainfer_amd._C.kernel.seq_mix import causal_conv
     g = torch.Generator().manual_seed(C + taps)
@@ -257,7 +257,10 @@ def _scan_reference(mode, q, k, v, decay, vscale, beta, bonus, H, G, K, V):
 @pytest.mark.parametrize("mode,H,G,K,V,per_channel", [("decay", 4, 2, 16, 8, False), ("decay", 3, 3, 7, 5, False), ("decay", 2, 1, 128, 64, False),
                                                       ("bonus", 3, 3, 16, 16, True), ("bonus", 1, 1, 9, 9, True), ("bonus", 2, 2, 64, 64, True),
                                                       ("delta", 4, 2, 16, 24, False), ("delta", 3, 3, 6, 10, False), ("delta", 2, 1, 130, 32, False),
-                                                      ("delta", 1, 1, 40, 200, False), ("decay", 2, 2, 24, 40, True)])
+                                                      ("delta", 1, 1, 40, 200, False), ("decay", 2, 2, 24, 40, True),
+                                                      # enough heads that a launch of prompts fills the chip: the layouts of large launches
+                                                      ("decay", 130, 65, 128, 32, False), ("bonus", 132, 132, 64, 32, True),
+                                                      ("delta", 134, 67, 72, 32, False)])
 def test_state_scan_forms_sizes_portions_and_slots(mode, H, G, K, V, per_channel):
     from hydrainfer_amd._C.kernel.seq_mix import state_scan
     g = torch.Generator().manual_seed(H * K + V)
