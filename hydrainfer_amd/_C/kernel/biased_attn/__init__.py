@@ -64,15 +64,17 @@ def qk_norm_cache(proj: Tensor, q_size: int, k_size: int, v_size: int, q_w: Opti
 def biased_attention(q: Tensor, key_cache: Tensor, value_cache: Tensor, vdim: int, tok_seq: Tensor, positions: Tensor,
                      q_cu: Tensor, block_table: Tensor, cu_block_lens: Tensor, scale: float,
                      slopes: Optional[Tensor] = None, mask: str = "causal", mask_size: int = 0, max_q_len: int = 0,
-                     kv_heads: Optional[int] = None, max_kv_len: int = 0, form: str = "auto", softcap: float = 0.0) -> Tensor:
+                     kv_heads: Optional[int] = None, max_kv_len: int = 0, form: str = "auto", softcap: float = 0.0,
+                     head_scale: Optional[Tensor] = None, sinks: Optional[Tensor] = None) -> Tensor:
     """q: [n_tokens, n_heads, dim] contiguous.  kv_heads: the key / value heads in use (the first of every cache row;
     default: all the plane has).  max_q_len: the longest portion of the batch; max_kv_len: the most keys a sequence holds —
     with few rows in the launch (decode steps) the keys of every tile are dealt to several waves.  form: "auto" (bfloat16
     with sizes that are multiples of 8: the MFMA forms — portions of prompts share every chunk of keys between four row
     tiles, decode steps split the keys), "tile" (the MFMA tile form throughout) or "rows" (one wave per token and head, any
-    dtype and size).
+    dtype and size).  head_scale [n_heads]: head h's scores are multiplied by head_scale[h] as well (a temperature per head);
+    sinks [n_heads]: the softmax's denominator of head h holds one more term exp(sinks[h]) without a key or a value.
     Returns [n_tokens, n_heads, vdim]."""
-    _lib.require_gpu(q, key_cache, value_cache, tok_seq, positions, q_cu, block_table, cu_block_lens, slopes)
+    _lib.require_gpu(q, key_cache, value_cache, tok_seq, positions, q_cu, block_table, cu_block_lens, slopes, head_scale, sinks)
     if q.dim() != 3 or not q.is_contiguous() or key_cache.dtype != q.dtype or value_cache.dtype != q.dtype:
         raise _lib.HydraHipError("biased_attention: q contiguous [n_tokens, n_heads, dim], caches of the same dtype")
     T, H, D = q.shape
@@ -89,10 +91,15 @@ def biased_attention(q: Tensor, key_cache: Tensor, value_cache: Tensor, vdim: in
             raise _lib.HydraHipError(f"biased_attention: {name} must be contiguous int32 [{n}]")
     if slopes is not None and (slopes.dtype != torch.float32 or not slopes.is_contiguous() or slopes.numel() != H):
         raise _lib.HydraHipError("biased_attention: slopes must be contiguous float32 [n_heads]")
+    for w, name in ((head_scale, "head_scale"), (sinks, "sinks")):
+        if w is not None and (w.dtype != torch.float32 or not w.is_contiguous() or w.numel() != H):
+            raise _lib.HydraHipError(f"biased_attention: {name} must be contiguous float32 [n_heads]")
     if mask not in MASK_KINDS or (mask != "causal" and mask_size < 1):
         raise _lib.HydraHipError(f"biased_attention: mask {mask!r} of size {mask_size}")
     out = torch.empty((T, H, vdim), dtype=q.dtype, device=q.device)
     a = _lib.hxm_biased_attn_args()
+    a.head_scale = None if head_scale is None else head_scale.data_ptr()
+    a.sinks = None if sinks is None else sinks.data_ptr()
     a.out, a.q, a.key_cache, a.value_cache = out.data_ptr(), q.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr()
     a.slopes = None if slopes is None else slopes.data_ptr()
     a.tok_seq, a.positions, a.q_cu = tok_seq.data_ptr(), positions.data_ptr(), q_cu.data_ptr()

@@ -49,11 +49,13 @@ def latent_norm_cache(proj: Tensor, q_off: int, q_rank: int, kv_off: int, kv_ran
 
 def latent_attention(q: Tensor, cache: Tensor, tok_seq: Tensor, positions: Tensor, q_cu: Tensor, block_table: Tensor,
                      cu_block_lens: Tensor, scale: float, window: Optional[int], max_q_len: int,
-                     gate_pre: Optional[Tensor] = None, out: Optional[Tensor] = None, max_kv_len: int = 0) -> Tensor:
+                     gate_pre: Optional[Tensor] = None, out: Optional[Tensor] = None, max_kv_len: int = 0,
+                     sinks: Optional[Tensor] = None) -> Tensor:
     """q: [n_tokens, n_heads, kv_rank] (any token / head strides, contiguous rows).  max_kv_len: the most keys a sequence
     of the batch holds — lets a launch with few rows (decode steps) deal every row tile's keys to several waves.  gate_pre [n_tokens, >= n_heads]:
-    the result of head h is multiplied by sigmoid(gate_pre[t, h]).  Returns [n_tokens, n_heads, kv_rank]."""
-    _lib.require_gpu(q, cache, tok_seq, positions, q_cu, block_table, cu_block_lens, gate_pre, out)
+    the result of head h is multiplied by sigmoid(gate_pre[t, h]).  sinks [n_heads] float32: the softmax's denominator of
+    head h holds one more term exp(sinks[h]) without a key or a value.  Returns [n_tokens, n_heads, kv_rank]."""
+    _lib.require_gpu(q, cache, tok_seq, positions, q_cu, block_table, cu_block_lens, gate_pre, out, sinks)
     if q.dim() != 3 or q.stride(2) != 1 or cache.dtype != q.dtype:
         raise _lib.HydraHipError("latent_attention: q [n_tokens, n_heads, kv_rank] with contiguous rows, cache of the same dtype")
     T, H, R = q.shape
@@ -68,7 +70,10 @@ def latent_attention(q: Tensor, cache: Tensor, tok_seq: Tensor, positions: Tenso
         out = torch.empty((T, H, R), dtype=q.dtype, device=q.device)
     elif out.shape != q.shape or out.dtype != q.dtype or out.stride(2) != 1:
         raise _lib.HydraHipError("latent_attention: out must look like q")
+    if sinks is not None and (sinks.dtype != torch.float32 or not sinks.is_contiguous() or sinks.numel() != H):
+        raise _lib.HydraHipError("latent_attention: sinks must be contiguous float32 [n_heads]")
     a = _lib.hxm_latent_attn_args()
+    a.sinks = None if sinks is None else sinks.data_ptr()
     a.out, a.q, a.cache = out.data_ptr(), q.data_ptr(), cache.data_ptr()
     a.gate_pre = None
     a.gate_stride = 0

@@ -16,9 +16,10 @@ def _code(dtype: torch.dtype) -> int:
 
 
 def route_softmax_topk(logits: Tensor, n_experts: int, top: int, scale: float,
-                       choice_bias: Optional[Tensor] = None) -> Tuple[Tensor, Tensor]:
+                       choice_bias: Optional[Tensor] = None, renorm: bool = True) -> Tuple[Tensor, Tensor]:
     """logits: float32 [n_tokens, >= n_experts] (contiguous rows).  s = softmax(logits[:, :n_experts]); the `top` largest of
-    s + choice_bias are chosen (ties: the lower expert); weights = chosen s / (their sum + 1e-20) * scale.
+    s + choice_bias are chosen (ties: the lower expert); weights = chosen s / (their sum + 1e-20) * scale, or with
+    renorm=False the chosen scores themselves, s * scale.
     Returns (weights float32 [n_tokens, top], experts int32 [n_tokens, top])."""
     _lib.require_gpu(logits, choice_bias)
     if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1 or logits.shape[1] < n_experts:
@@ -31,7 +32,8 @@ def route_softmax_topk(logits: Tensor, n_experts: int, top: int, scale: float,
     experts = torch.empty((T, top), dtype=torch.int32, device=logits.device)
     _lib.mix_check(_lib.mix_lib().hxm_route_softmax_topk(
         logits.data_ptr(), logits.stride(0), None if choice_bias is None else choice_bias.data_ptr(), T, int(n_experts),
-        int(top), float(scale), weights.data_ptr(), experts.data_ptr(), _lib.current_stream()), "route_softmax_topk")
+        int(top), float(scale), 1 if renorm else 0, weights.data_ptr(), experts.data_ptr(), _lib.current_stream()),
+        "route_softmax_topk")
     return weights, experts
 
 
@@ -72,10 +74,12 @@ def grouped_linear(x: Tensor, w: Tensor, seg: Tensor, max_rows: int, src: Option
 
 
 def moe_combine(y: Tensor, row_of: Tensor, weights: Tensor, shared: Optional[Tensor] = None,
-                shared_gate: Optional[Tensor] = None) -> Tensor:
+                shared_gate: Optional[Tensor] = None, identity: Optional[Tensor] = None) -> Tensor:
     """out[t] = sum_k weights[t, k] * y[row_of[t, k]] + sigmoid(shared_gate[t]) * shared[t].  shared_gate: float32, one
-    number per token (any row stride: a column of a wider matrix will do)."""
-    _lib.require_gpu(y, row_of, weights, shared, shared_gate)
+    number per token (any row stride: a column of a wider matrix will do).  identity [n_tokens, width] (the experts' input):
+    a choice without a row (row_of < 0: an expert beyond those moe_plan was called with) is an identity expert and adds
+    weights[t, k] * identity[t]; without it such a choice adds nothing."""
+    _lib.require_gpu(y, row_of, weights, shared, shared_gate, identity)
     T, top = row_of.shape
     W = y.shape[1]
     if y.dim() != 2 or not y.is_contiguous() or weights.dtype != torch.float32 or not weights.is_contiguous() or \
@@ -87,9 +91,12 @@ def moe_combine(y: Tensor, row_of: Tensor, weights: Tensor, shared: Optional[Ten
                 shared_gate.dtype != torch.float32 or shared_gate.shape[0] != T:
             raise _lib.HydraHipError("moe_combine: shared [n_tokens, width] of y's dtype with a float32 gate per token")
         gate_stride = shared_gate.stride(0)
+    if identity is not None and (identity.dtype != y.dtype or identity.dim() != 2 or identity.shape[0] != T or
+                                 identity.shape[1] < W or identity.stride(1) != 1):
+        raise _lib.HydraHipError("moe_combine: identity must be [n_tokens, >= width] of y's dtype with contiguous rows")
     out = torch.empty((T, W), dtype=y.dtype, device=y.device)
     _lib.mix_check(_lib.mix_lib().hxm_moe_combine(
         out.data_ptr(), y.data_ptr(), row_of.data_ptr(), weights.data_ptr(), None if shared is None else shared.data_ptr(),
-        None if shared is None else shared_gate.data_ptr(), gate_stride, T, top, W, _code(y.dtype), _lib.current_stream()),
-        "moe_combine")
+        None if shared is None else shared_gate.data_ptr(), gate_stride, None if identity is None else identity.data_ptr(),
+        0 if identity is None else identity.stride(0), T, top, W, _code(y.dtype), _lib.current_stream()), "moe_combine")
     return out

@@ -87,6 +87,32 @@ def causal_conv(u: Tensor, w: Tensor, bias: Optional[Tensor], act: Optional[str]
     return y
 
 
+def causal_conv_pair(u: Tensor, w: Tensor, w2: Optional[Tensor], seq: SequenceState, offset: int, q_cu: Tensor, positions: Tensor,
+                     bias: Optional[Tensor] = None, bias2: Optional[Tensor] = None, act: Optional[str] = None,
+                     skip: bool = True):
+    """Two short causal convolutions of the same input in one pass: y = act(conv_w(u) + bias) + u, y2 = act(conv_w2(u) +
+    bias2) + u (skip=False: without the + u).  The inputs are read once and the slot's piece ((taps - 1) * channels floats,
+    the inputs of the last positions) is brought up to date once.  w2 None: only y.  Returns (y, y2 or None)."""
+    _lib.require_gpu(u, w, w2, bias, bias2)
+    if u.dim() != 2 or u.stride(1) != 1:
+        raise _lib.HydraHipError("causal_conv_pair: u must be 2-D with contiguous rows")
+    T, C = u.shape
+    if w.dim() != 2 or w.shape[0] != C or (w2 is not None and w2.shape != w.shape):
+        raise _lib.HydraHipError("causal_conv_pair: w and w2 must be [channels, taps]")
+    taps = w.shape[1]
+    _f32(w, C * taps, "causal_conv_pair: w"); _f32(w2, C * taps, "causal_conv_pair: w2")
+    _f32(bias, C, "causal_conv_pair: bias"); _f32(bias2, C, "causal_conv_pair: bias2")
+    n_seq = _batch(seq, q_cu, positions, T, "causal_conv_pair")
+    base, stride = _piece(seq, offset, max(taps - 1, 1) * C, "causal_conv_pair")
+    y = torch.empty((T, C), dtype=u.dtype, device=u.device)
+    y2 = torch.empty((T, C), dtype=u.dtype, device=u.device) if w2 is not None else None
+    _lib.mix_check(_lib.mix_lib().hxm_causal_conv_pair(
+        y.data_ptr(), y.stride(0), _ptr(y2), C if y2 is not None else 0, u.data_ptr(), u.stride(0), w.data_ptr(), _ptr(w2),
+        _ptr(bias), _ptr(bias2), ACT[act], 1 if skip else 0, base, stride, seq.slots.data_ptr(), seq.tok_seq.data_ptr(),
+        q_cu.data_ptr(), positions.data_ptr(), T, n_seq, C, taps, _code(u.dtype), _lib.current_stream()), "causal_conv_pair")
+    return y, y2
+
+
 def token_shift_mix(h: Tensor, mu: Tensor, seq: SequenceState, offset: int, q_cu: Tensor, positions: Tensor) -> Tensor:
     """out[m] = h + (h_prev - h) * mu[m], h_prev the row of the token before in the same sequence (zeros before position 0).
     h: [n_tokens, width]; mu: float32 [n_mix, width]; the slot's piece: width floats.  Returns [n_mix, n_tokens, width]."""

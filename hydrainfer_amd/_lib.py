@@ -211,7 +211,7 @@ def lib() -> ctypes.CDLL:
 # a paged latent cache.  A library of its own, so that a model that needs only these builds only these (`make mix`).
 # ---------------------------------------------------------------------------------------------------------
 MIX_LIB_PATH = os.environ.get("HX_MIX_LIB_PATH") or os.path.join(_HERE, "lib", "libhydra_mix.so")
-HXM_ABI_VERSION = 3
+HXM_ABI_VERSION = 4
 HXM_MAX_STREAMS = 16
 HXM_MAX_LATENT = 1024
 
@@ -226,7 +226,7 @@ class hxm_latent_attn_args(ctypes.Structure):
         ("cache_row_stride", c_int64),
         ("n_tokens", c_int32), ("n_seq", c_int32), ("n_heads", c_int32), ("kv_rank", c_int32), ("block_size", c_int32),
         ("window", c_int32), ("max_q_len", c_int32), ("scale", c_float), ("dtype", c_int32),
-        ("max_kv_len", c_int32), ("n_splits", c_int32), ("ws_o", c_void_p), ("ws_ml", c_void_p),
+        ("max_kv_len", c_int32), ("n_splits", c_int32), ("ws_o", c_void_p), ("ws_ml", c_void_p), ("sinks", c_void_p),
     ]
 
 
@@ -236,6 +236,7 @@ class hxm_depth_norm_args(ctypes.Structure):
         ("depth_w", c_void_p), ("x_out", c_void_p), ("next_w", c_void_p), ("h_out", c_void_p), ("rows", c_void_p),
         ("y_stride", c_int64), ("level_stride", c_int64), ("n_out", c_int64), ("width", c_int64),
         ("n_levels", c_int32), ("rms", c_int32), ("dtype", c_int32), ("mult", c_float), ("eps", c_float),
+        ("y2", c_void_p), ("bias", c_void_p), ("y2_stride", c_int64), ("h_stride", c_int64), ("post_norm", c_int32),
     ]
 
 
@@ -247,7 +248,7 @@ class hxm_biased_attn_args(ctypes.Structure):
         ("n_tokens", c_int32), ("n_heads", c_int32), ("kv_heads", c_int32), ("dim", c_int32), ("vdim", c_int32),
         ("block_size", c_int32), ("mask_kind", c_int32), ("mask_size", c_int32), ("scale", c_float), ("dtype", c_int32),
         ("q_cu", c_void_p), ("n_seq", c_int32), ("max_q_len", c_int32), ("form", c_int32), ("n_splits", c_int32),
-        ("ws_o", c_void_p), ("ws_ml", c_void_p), ("softcap", c_float),
+        ("ws_o", c_void_p), ("ws_ml", c_void_p), ("softcap", c_float), ("head_scale", c_void_p), ("sinks", c_void_p),
     ]
 
 
@@ -258,6 +259,23 @@ class hxm_head_rope_args(ctypes.Structure):
         ("key_cache", c_void_p), ("value_cache", c_void_p), ("cache_row_stride", c_int64), ("head_stride", c_int64),
         ("n_tokens", c_int64), ("q_heads", c_int32), ("kv_heads", c_int32), ("dim", c_int32), ("rot_dims", c_int32),
         ("eps", c_float), ("cos_sin_scale", c_float), ("dtype", c_int32),
+    ]
+
+
+class hxm_rotary_part(ctypes.Structure):
+    _fields_ = [
+        ("src", c_void_p), ("dst", c_void_p), ("inv_freq", c_void_p), ("gate", c_void_p),
+        ("src_stride", c_int64), ("src_head_stride", c_int64), ("dst_stride", c_int64), ("dst_head_stride", c_int64),
+        ("cache_block_stride", c_int64), ("gate_stride", c_int64),
+        ("heads", c_int32), ("size", c_int32), ("rot_off", c_int32), ("rot_dims", c_int32), ("layout", c_int32),
+        ("to_cache", c_int32), ("gate_kind", c_int32), ("mag", c_float), ("sign", c_float),
+    ]
+
+
+class hxm_rotary_args(ctypes.Structure):
+    _fields_ = [
+        ("parts", hxm_rotary_part * 3), ("positions", c_void_p), ("slot_ids", c_void_p), ("n_tokens", c_int64),
+        ("n_parts", c_int32), ("block_size", c_int32), ("dtype", c_int32),
     ]
 
 
@@ -304,12 +322,13 @@ _MIX_SIGNATURES = {
     "hxm_depth_norm": (c_int, [POINTER(hxm_depth_norm_args), c_void_p]),
     "hxm_poly_norm": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_float, c_int64, c_int64, c_int, c_void_p]),
     "hxm_relu_squared": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
-    "hxm_route_softmax_topk": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int32, c_int32, c_float, c_void_p, c_void_p, c_void_p]),
+    "hxm_route_softmax_topk": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int32, c_int32, c_float, c_int32, c_void_p, c_void_p,
+                                       c_void_p]),
     "hxm_moe_plan": (c_int, [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]),
     "hxm_grouped_linear": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int64, c_int64,
                                    c_int32, c_int, c_void_p]),
-    "hxm_moe_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int64,
-                                c_int, c_void_p]),
+    "hxm_moe_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int64,
+                                c_int32, c_int64, c_int, c_void_p]),
     "hxm_gated_recurrence_workspace": (c_int64, [c_int64, c_int32, c_int32, c_int32]),
     "hxm_gated_recurrence": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
                                      c_float, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32,
@@ -320,6 +339,10 @@ _MIX_SIGNATURES = {
     "hxm_biased_attention": (c_int, [POINTER(hxm_biased_attn_args), c_void_p]),
     "hxm_causal_conv": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_void_p,
                                 c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_int32, c_int, c_void_p]),
+    "hxm_causal_conv_pair": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
+                                     c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int32,
+                                     c_int32, c_int32, c_int, c_void_p]),
+    "hxm_rotary_parts": (c_int, [POINTER(hxm_rotary_args), c_void_p]),
     "hxm_token_shift_mix": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_int32, c_void_p, c_int64, c_void_p, c_void_p,
                                     c_void_p, c_void_p, c_int64, c_int32, c_int64, c_int, c_void_p]),
     "hxm_clamped_glu": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_float, c_float, c_float, c_int64,

@@ -132,7 +132,8 @@ __global__ __launch_bounds__(256) void biased_attn_rows_kernel(hxm_biased_attn_a
   float* qs = lds + wave * (D + 64);       // the query, then the group's weights
   float* ps = qs + D;
   const T* q = (const T*)a.q + ((int64_t)t * a.n_heads + h) * D;
-  for (int d = lane; d < D; d += 64) qs[d] = A::to_float(q[d]) * a.scale;
+  const float qscale = a.head_scale ? a.scale * a.head_scale[h] : a.scale;
+  for (int d = lane; d < D; d += 64) qs[d] = A::to_float(q[d]) * qscale;
   wave_lds_sync();
   const int seq = a.tok_seq[t], i = a.positions[t];
   const int32_t* table = a.block_table + a.cu_block_lens[seq];
@@ -178,6 +179,7 @@ __global__ __launch_bounds__(256) void biased_attn_rows_kernel(hxm_biased_attn_a
     }
   }
   T* o = (T*)a.out + ((int64_t)t * a.n_heads + h) * V;
+  if (a.sinks) l += expf(a.sinks[h] - m);      // the sink: one more term of the denominator, without a value
   const float inv = 1.0f / l;
 #pragma unroll
   for (int c = 0; c < kMaxVCols; ++c) {
@@ -238,14 +240,19 @@ __global__ __launch_bounds__(256) void biased_attn_tile_kernel(hxm_biased_attn_a
   }
   // the rows this lane holds of S and O: 4 g + i
   int pos[4], lo[4];
-  float slope[4];
+  float slope[4], hsc[4], snk[4];      // per row: distance slope, score scale (scale * head_scale), sink term's logit
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = tile * 16 + 4 * g + i;
+    hsc[i] = a.scale;
+    snk[i] = -INFINITY;
     if (r < n_rows) {
+      const int h = kvh * R + r % R;
       pos[i] = a.positions[q0 + r / R];
       lo[i] = first_visible(pos[i], a.mask_kind, a.mask_size);
-      slope[i] = a.slopes ? a.slopes[kvh * R + r % R] : 0.f;
+      slope[i] = a.slopes ? a.slopes[h] : 0.f;
+      if (a.head_scale) hsc[i] = a.scale * a.head_scale[h];
+      if (a.sinks) snk[i] = a.sinks[h];
     } else {
       pos[i] = -1;      // sees nothing
       lo[i] = 0;
@@ -317,7 +324,7 @@ __global__ __launch_bounds__(256) void biased_attn_tile_kernel(hxm_biased_attn_a
       for (int s = 0; s < 2; ++s) {
         const int key = key0 + 16 * s + c;
         const bool seen = key >= lo[i] && key <= pos[i];
-        p[s] = seen ? capped(sc[s][i] * a.scale, a.softcap) - slope[i] * (float)(pos[i] - key) : -INFINITY;
+        p[s] = seen ? capped(sc[s][i] * hsc[i], a.softcap) - slope[i] * (float)(pos[i] - key) : -INFINITY;
         mx = fmaxf(mx, p[s]);
       }
       mx = row16_max(mx);      // (the sixteen lanes that hold the row's scores: one DPP row)
@@ -381,7 +388,7 @@ __global__ __launch_bounds__(256) void biased_attn_tile_kernel(hxm_biased_attn_a
   for (int i = 0; i < 4; ++i) {
     const int r = tile * 16 + 4 * g + i;
     if (r >= n_rows) continue;
-    const float inv = 1.0f / l[i];
+    const float inv = 1.0f / (l[i] + expf(snk[i] - m[i]));      // (no sink: exp(-inf) = 0)
     u16* og = (u16*)a.out + ((int64_t)(q0 + r / R) * a.n_heads + kvh * R + r % R) * V;
 #pragma unroll
     for (int n = 0; n < KK * 2; ++n) {
@@ -438,14 +445,19 @@ __global__ __launch_bounds__(256) void biased_attn_group_kernel(hxm_biased_attn_
     }
   }
   int pos[4], lo[4];
-  float slope[4];
+  float slope[4], hsc[4], snk[4];      // per row: distance slope, score scale (scale * head_scale), sink term's logit
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = tile * 16 + 4 * g + i;
+    hsc[i] = a.scale;
+    snk[i] = -INFINITY;
     if (r < n_rows) {
+      const int h = kvh * R + r % R;
       pos[i] = a.positions[q0 + r / R];
       lo[i] = first_visible(pos[i], a.mask_kind, a.mask_size);
-      slope[i] = a.slopes ? a.slopes[kvh * R + r % R] : 0.f;
+      slope[i] = a.slopes ? a.slopes[h] : 0.f;
+      if (a.head_scale) hsc[i] = a.scale * a.head_scale[h];
+      if (a.sinks) snk[i] = a.sinks[h];
     } else {
       pos[i] = -1;      // sees nothing
       lo[i] = 0;
@@ -522,7 +534,7 @@ __global__ __launch_bounds__(256) void biased_attn_group_kernel(hxm_biased_attn_
         for (int s = 0; s < 2; ++s) {
           const int key = key0 + 16 * s + c;
           const bool seen = key >= lo[i] && key <= pos[i];
-          p[s] = seen ? capped(sc[s][i] * a.scale, a.softcap) - slope[i] * (float)(pos[i] - key) : -INFINITY;
+          p[s] = seen ? capped(sc[s][i] * hsc[i], a.softcap) - slope[i] * (float)(pos[i] - key) : -INFINITY;
           mx = fmaxf(mx, p[s]);
         }
         mx = row16_max(mx);
@@ -563,7 +575,7 @@ __global__ __launch_bounds__(256) void biased_attn_group_kernel(hxm_biased_attn_
   for (int i = 0; i < 4; ++i) {
     const int r = tile * 16 + 4 * g + i;
     if (r >= n_rows) continue;
-    const float inv = 1.0f / l[i];
+    const float inv = 1.0f / (l[i] + expf(snk[i] - m[i]));      // (no sink: exp(-inf) = 0)
     u16* og = (u16*)a.out + ((int64_t)(q0 + r / R) * a.n_heads + kvh * R + r % R) * V;
 #pragma unroll
     for (int n = 0; n < KK * 2; ++n) {
@@ -591,6 +603,7 @@ __global__ __launch_bounds__(256) void biased_attn_combine_kernel(hxm_biased_att
     for (int s = 0; s < NS; ++s) M = fmaxf(M, wml[s * 32 + 2 * row]);
     float L = 0.f;
     for (int s = 0; s < NS; ++s) L += wml[s * 32 + 2 * row + 1] * __expf(wml[s * 32 + 2 * row] - M);
+    if (a.sinks) L += expf(a.sinks[kvh * R + (tile * 16 + row) % R] - M);      // the sink counts once, here
     const float inv = L > 0.f ? 1.0f / L : 0.f;
     for (int s = 0; s < NS; ++s) wgt[row][s] = __expf(wml[s * 32 + 2 * row] - M) * inv;
   }

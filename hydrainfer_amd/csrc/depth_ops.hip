@@ -68,16 +68,26 @@ __global__ __launch_bounds__(256) void depth_norm_kernel(hxm_depth_norm_args a) 
   typedef typename A::storage T;
   const int64_t W = a.width, i_out = blockIdx.x;
   const int64_t r = a.rows ? (int64_t)a.rows[i_out] : i_out;
-  const float* xin = a.x_in + r * W;
+  const float* xin = a.x_in ? a.x_in + r * W : nullptr;
   if (a.y) {
     const T* y = (const T*)a.y + r * a.y_stride;
     for (int64_t i = threadIdx.x; i < W; i += 256) buf[i] = A::to_float(y[i]);
-    __syncthreads();
-    float shift, inv;
-    row_stats(buf, part, W, a.eps, a.rms, shift, inv);
-    for (int64_t i = threadIdx.x; i < W; i += 256) buf[i] = xin[i] + a.mult * ((buf[i] - shift) * inv * a.post_w[i]);
+    float shift = 0.f, inv = 1.f;
+    if (a.post_norm != HXM_POST_PLAIN) {
+      __syncthreads();
+      row_stats(buf, part, W, a.eps, a.post_norm == HXM_POST_SAME ? a.rms : a.post_norm == HXM_POST_RMS, shift, inv);
+    }
+    for (int64_t i = threadIdx.x; i < W; i += 256)
+      buf[i] = (xin ? xin[i] : 0.f) + a.mult * ((buf[i] - shift) * inv * (a.post_w ? a.post_w[i] : 1.f));
   } else {
-    for (int64_t i = threadIdx.x; i < W; i += 256) buf[i] = xin[i];
+    for (int64_t i = threadIdx.x; i < W; i += 256) buf[i] = xin ? xin[i] : 0.f;
+  }
+  if (a.y2) {
+    const T* y2 = (const T*)a.y2 + r * a.y2_stride;
+    for (int64_t i = threadIdx.x; i < W; i += 256) buf[i] += A::to_float(y2[i]);
+  }
+  if (a.bias) {
+    for (int64_t i = threadIdx.x; i < W; i += 256) buf[i] += a.bias[i];
   }
   // (every thread keeps to the elements i = tid + 256 k from here on: no barrier is needed until the next statistics)
   if (a.level_out) {
@@ -104,8 +114,11 @@ __global__ __launch_bounds__(256) void depth_norm_kernel(hxm_depth_norm_args a) 
     __syncthreads();
     float shift, inv;
     row_stats(buf, part, W, a.eps, a.rms, shift, inv);
-    T* h = (T*)a.h_out + i_out * W;
+    T* h = (T*)a.h_out + i_out * a.h_stride;
     for (int64_t i = threadIdx.x; i < W; i += 256) h[i] = A::from_float((buf[i] - shift) * inv * a.next_w[i]);
+  } else if (a.h_out) {      // no norm: the row itself in the activations' type
+    T* h = (T*)a.h_out + i_out * a.h_stride;
+    for (int64_t i = threadIdx.x; i < W; i += 256) h[i] = A::from_float(buf[i]);
   }
 }
 
@@ -141,23 +154,46 @@ __global__ __launch_bounds__(256) void depth_norm_vec_kernel(hxm_depth_norm_args
   typedef typename A::storage T;
   const int64_t W = a.width, n4 = W >> 2, i_out = blockIdx.x;
   const int64_t r = a.rows ? (int64_t)a.rows[i_out] : i_out;
-  const f32x4* xin = reinterpret_cast<const f32x4*>(a.x_in + r * W);
+  const f32x4* xin = a.x_in ? reinterpret_cast<const f32x4*>(a.x_in + r * W) : nullptr;
+  const f32x4 zero4 = f32x4{0.f, 0.f, 0.f, 0.f}, one4 = f32x4{1.f, 1.f, 1.f, 1.f};
   if (a.y) {
     const T* y = (const T*)a.y + r * a.y_stride;
     for (int64_t i = threadIdx.x; i < n4; i += 256) buf[i] = Row4<A>::load(y + 4 * i);
-    __syncthreads();
-    float shift, inv;
-    row_stats4(lds, part, W, a.eps, a.rms, shift, inv);
+    float shift = 0.f, inv = 1.f;
+    if (a.post_norm != HXM_POST_PLAIN) {
+      __syncthreads();
+      row_stats4(lds, part, W, a.eps, a.post_norm == HXM_POST_SAME ? a.rms : a.post_norm == HXM_POST_RMS, shift, inv);
+    }
     const f32x4* pw = reinterpret_cast<const f32x4*>(a.post_w);
     for (int64_t i = threadIdx.x; i < n4; i += 256) {
-      const f32x4 v = buf[i], x = xin[i], w = pw[i];
+      const f32x4 v = buf[i], x = xin ? xin[i] : zero4, w = pw ? pw[i] : one4;
       f32x4 o;
 #pragma unroll
       for (int k = 0; k < 4; ++k) o[k] = x[k] + a.mult * ((v[k] - shift) * inv * w[k]);
       buf[i] = o;
     }
   } else {
-    for (int64_t i = threadIdx.x; i < n4; i += 256) buf[i] = xin[i];
+    for (int64_t i = threadIdx.x; i < n4; i += 256) buf[i] = xin ? xin[i] : zero4;
+  }
+  if (a.y2) {
+    const T* y2 = (const T*)a.y2 + r * a.y2_stride;
+    for (int64_t i = threadIdx.x; i < n4; i += 256) {
+      const f32x4 v = Row4<A>::load(y2 + 4 * i);
+      f32x4 o = buf[i];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) o[k] += v[k];
+      buf[i] = o;
+    }
+  }
+  if (a.bias) {
+    const f32x4* bw = reinterpret_cast<const f32x4*>(a.bias);
+    for (int64_t i = threadIdx.x; i < n4; i += 256) {
+      const f32x4 v = bw[i];
+      f32x4 o = buf[i];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) o[k] += v[k];
+      buf[i] = o;
+    }
   }
   // (every thread keeps to the elements i = tid + 256 k from here on: no barrier is needed until the next statistics)
   if (a.level_out) {
@@ -186,7 +222,7 @@ __global__ __launch_bounds__(256) void depth_norm_vec_kernel(hxm_depth_norm_args
     __syncthreads();
     float shift, inv;
     row_stats4(lds, part, W, a.eps, a.rms, shift, inv);
-    T* h = (T*)a.h_out + i_out * W;
+    T* h = (T*)a.h_out + i_out * a.h_stride;
     const f32x4* nw = reinterpret_cast<const f32x4*>(a.next_w);
     for (int64_t i = threadIdx.x; i < n4; i += 256) {
       const f32x4 v = buf[i], w = nw[i];
@@ -195,6 +231,9 @@ __global__ __launch_bounds__(256) void depth_norm_vec_kernel(hxm_depth_norm_args
       for (int k = 0; k < 4; ++k) o[k] = (v[k] - shift) * inv * w[k];
       Row4<A>::store(h + 4 * i, o);
     }
+  } else if (a.h_out) {      // no norm: the row itself in the activations' type
+    T* h = (T*)a.h_out + i_out * a.h_stride;
+    for (int64_t i = threadIdx.x; i < n4; i += 256) Row4<A>::store(h + 4 * i, buf[i]);
   }
 }
 
@@ -291,8 +330,10 @@ extern "C" int hxm_depth_norm(const hxm_depth_norm_args* args, void* stream) {
   const hxm_depth_norm_args& a = *args;
   if (a.n_out < 0 || a.width < 1 || a.n_levels < 0) return HX_ERR_SHAPE;
   if (a.n_out == 0) return HX_OK;
-  if (!a.x_in || (a.y && !a.post_w) || (a.depth_w && !a.levels) || (a.next_w && !a.h_out)) return HX_ERR_NULL;
-  if (a.y && a.y_stride < a.width) return HX_ERR_STRIDE;
+  if (a.post_norm < HXM_POST_SAME || a.post_norm > HXM_POST_PLAIN) return HX_ERR_SHAPE;
+  if ((!a.x_in && !a.y) || (a.y && !a.post_w && a.post_norm != HXM_POST_PLAIN) || (a.depth_w && !a.levels) || (a.next_w && !a.h_out))
+    return HX_ERR_NULL;
+  if ((a.y && a.y_stride < a.width) || (a.y2 && a.y2_stride < a.width) || (a.h_out && a.h_stride < a.width)) return HX_ERR_STRIDE;
   const size_t lds = ((size_t)a.width + 4) * sizeof(float);
   if (lds > 64 * 1024) return HX_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
@@ -301,7 +342,8 @@ extern "C" int hxm_depth_norm(const hxm_depth_norm_args* args, void* stream) {
   auto by16 = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
   const bool vec = a.width % 4 == 0 && by16(a.x_in) && by16(a.post_w) && by16(a.level_out) && by16(a.levels) && a.level_stride % 4 == 0 &&
                    by16(a.x_out) && by16(a.next_w) && ((uintptr_t)a.y % (4 * es)) == 0 && a.y_stride % 4 == 0 &&
-                   ((uintptr_t)a.h_out % (4 * es)) == 0;
+                   ((uintptr_t)a.h_out % (4 * es)) == 0 && a.h_stride % 4 == 0 && ((uintptr_t)a.y2 % (4 * es)) == 0 &&
+                   a.y2_stride % 4 == 0 && by16(a.bias);
   switch (a.dtype) {
     case HX_F32:
       if (vec) depth_norm_vec_kernel<F32><<<grid, block, lds, s>>>(a);

@@ -139,6 +139,7 @@ __global__ __launch_bounds__(256) void latent_attn_rows_kernel(hxm_latent_attn_a
       }
     }
   }
+  if (a.sinks) l += expf(a.sinks[h] - m);      // the sink: one more term of the denominator, without a value
   float g = 1.0f / l;
   if (a.gate_pre) {
     const float z = A::to_float(((const typename A::storage*)a.gate_pre)[(int64_t)t * a.gate_stride + h]);
@@ -382,7 +383,7 @@ __global__ __launch_bounds__(256) void latent_attn_tile_kernel(hxm_latent_attn_a
     const int r = tile * 16 + 4 * g + i;
     if (r >= n_rows) continue;
     const int t = q0 + r / H, h = r % H;
-    float gsc = 1.0f / l[i];
+    float gsc = 1.0f / (a.sinks ? l[i] + expf(a.sinks[h] - m[i]) : l[i]);
     if (a.gate_pre) {
       const float z = BF16::to_float(((const u16*)a.gate_pre)[(int64_t)t * a.gate_stride + h]);
       gsc = gsc / (1.0f + __expf(-z));
@@ -585,7 +586,7 @@ __global__ __launch_bounds__(256) void latent_attn_tile_wide_kernel(hxm_latent_a
     const int r = tile * 16 + 4 * g + i;
     if (r >= n_rows) continue;
     const int t = q0 + r / H, h = r % H;
-    float gsc = 1.0f / l[i];
+    float gsc = 1.0f / (a.sinks ? l[i] + expf(a.sinks[h] - m[i]) : l[i]);
     if (a.gate_pre) {
       const float z = BF16::to_float(((const u16*)a.gate_pre)[(int64_t)t * a.gate_stride + h]);
       gsc = gsc / (1.0f + __expf(-z));
@@ -764,7 +765,7 @@ __global__ __launch_bounds__(256) void latent_attn_group_kernel(hxm_latent_attn_
     const int r = tile * 16 + 4 * g + i;
     if (r >= n_rows) continue;
     const int t = q0 + r / H, h = r % H;
-    float gsc = 1.0f / l[i];
+    float gsc = 1.0f / (a.sinks ? l[i] + expf(a.sinks[h] - m[i]) : l[i]);
     if (a.gate_pre) {
       const float z = BF16::to_float(((const u16*)a.gate_pre)[(int64_t)t * a.gate_stride + h]);
       gsc = gsc / (1.0f + __expf(-z));
@@ -795,6 +796,7 @@ __global__ __launch_bounds__(256) void latent_attn_combine_kernel(hxm_latent_att
     float L = 0.f;
     for (int s = 0; s < NS; ++s) L += wml[s * 32 + 2 * row + 1] * __expf(wml[s * 32 + 2 * row] - M);
     const int r = tile * 16 + row;
+    if (a.sinks && r < n_rows) L += expf(a.sinks[r % H] - M);      // the sink counts once, here
     float gsc = L > 0.f ? 1.0f / L : 0.f;
     if (a.gate_pre && r < n_rows) {
       const float z = BF16::to_float(((const u16*)a.gate_pre)[(int64_t)(q0 + r / H) * a.gate_stride + r % H]);
@@ -922,7 +924,8 @@ extern "C" int hxm_latent_attention(const hxm_latent_attn_args* args, void* stre
       case 4: return launch_tile<4>(a, s);
       case 5: case 6: return launch_tile<6>(a, s);
       case 7: case 8: return launch_tile<8>(a, s);
-      case 9: case 10: case 11: case 12: return launch_tile<12>(a, s);
+      case 9: case 10: return launch_tile<10>(a, s);
+      case 11: case 12: return launch_tile<12>(a, s);
       default: return launch_tile<16>(a, s);
     }
   }

@@ -23,7 +23,7 @@ template <int PER>
 __global__ __launch_bounds__(256) void route_softmax_topk_kernel(const float* __restrict__ logits, int64_t stride,
                                                                  const float* __restrict__ bias, int64_t n_tokens, int E,
                                                                  int top, float scale, float* __restrict__ weights,
-                                                                 int32_t* __restrict__ experts) {
+                                                                 int32_t* __restrict__ experts, int renorm) {
   const int lane = threadIdx.x & 63;
   const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= n_tokens) return;
@@ -88,7 +88,7 @@ __global__ __launch_bounds__(256) void route_softmax_topk_kernel(const float* __
     }
   }
   if (lane < top) {
-    weights[t * top + lane] = my_w / (chosen_sum + 1e-20f) * scale;
+    weights[t * top + lane] = (renorm ? my_w / (chosen_sum + 1e-20f) : my_w) * scale;
     experts[t * top + lane] = my_e;
   }
 }
@@ -298,15 +298,22 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(typename A::storage* _
                                                           const int32_t* __restrict__ row_of, const float* __restrict__ weights,
                                                           const typename A::storage* __restrict__ shared,
                                                           const float* __restrict__ shared_gate, int64_t gate_stride, int top,
-                                                          int64_t W) {
+                                                          int64_t W, const typename A::storage* __restrict__ identity,
+                                                          int64_t identity_stride) {
   const int64_t t = blockIdx.x;
   const float g = shared ? 1.0f / (1.0f + expf(-shared_gate[t * gate_stride])) : 0.f;
+  // a choice without a row (an expert past those the plan was made for) is an identity expert when `identity` is given
+  float idw = 0.f;
+  if (identity)
+    for (int k = 0; k < top; ++k)
+      if (row_of[t * top + k] < 0) idw += weights[t * top + k];
   for (int64_t i = threadIdx.x; i < W; i += 256) {
     float u = 0.f;
     for (int k = 0; k < top; ++k) {
       const int32_t r = row_of[t * top + k];
       if (r >= 0) u += weights[t * top + k] * A::to_float(y[(int64_t)r * W + i]);
     }
+    if (idw != 0.f) u += idw * A::to_float(identity[t * identity_stride + i]);
     if (shared) u += g * A::to_float(shared[t * W + i]);
     out[t * W + i] = A::from_float(u);
   }
@@ -315,8 +322,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(typename A::storage* _
 }  // namespace
 
 extern "C" int hxm_route_softmax_topk(const float* logits, int64_t logit_stride, const float* choice_bias, int64_t n_tokens,
-                                      int32_t n_experts, int32_t top, float scale, float* weights, int32_t* experts,
-                                      void* stream) {
+                                      int32_t n_experts, int32_t top, float scale, int32_t renorm, float* weights,
+                                      int32_t* experts, void* stream) {
   if (n_tokens < 0 || n_experts < 1 || n_experts > kMaxExperts || top < 1 || top > n_experts || top > 64) return HX_ERR_SHAPE;
   if (n_tokens == 0) return HX_OK;
   if (!logits || !weights || !experts) return HX_ERR_NULL;
@@ -324,7 +331,7 @@ extern "C" int hxm_route_softmax_topk(const float* logits, int64_t logit_stride,
   const dim3 grid((unsigned)((n_tokens + 3) / 4)), block(256);
   hipStream_t s = (hipStream_t)stream;
 #define HXM_ROUTE(PER_) route_softmax_topk_kernel<PER_><<<grid, block, 0, s>>>(logits, logit_stride, choice_bias, n_tokens, \
-                                                                              n_experts, top, scale, weights, experts)
+                                                                              n_experts, top, scale, weights, experts, renorm)
   if (n_experts <= 64) HXM_ROUTE(1);
   else if (n_experts <= 128) HXM_ROUTE(2);
   else if (n_experts <= 256) HXM_ROUTE(4);
@@ -382,9 +389,10 @@ extern "C" int hxm_grouped_linear(void* y, const void* x, int64_t x_stride, cons
 }
 
 extern "C" int hxm_moe_combine(void* out, const void* y, const int32_t* row_of, const float* weights, const void* shared,
-                               const float* shared_gate, int64_t gate_stride, int64_t n_tokens, int32_t top, int64_t width,
-                               int dtype, void* stream) {
+                               const float* shared_gate, int64_t gate_stride, const void* identity, int64_t identity_stride,
+                               int64_t n_tokens, int32_t top, int64_t width, int dtype, void* stream) {
   if (n_tokens < 0 || top < 1 || width < 1) return HX_ERR_SHAPE;
+  if (identity && identity_stride < width) return HX_ERR_STRIDE;
   if (n_tokens == 0) return HX_OK;
   if (!out || !y || !row_of || !weights || (shared && !shared_gate)) return HX_ERR_NULL;
   hipStream_t s = (hipStream_t)stream;
@@ -392,11 +400,11 @@ extern "C" int hxm_moe_combine(void* out, const void* y, const int32_t* row_of, 
   switch (dtype) {
     case HX_F32:
       moe_combine_kernel<F32><<<grid, block, 0, s>>>((float*)out, (const float*)y, row_of, weights, (const float*)shared, shared_gate,
-                                                     gate_stride, top, width);
+                                                     gate_stride, top, width, (const float*)identity, identity_stride);
       break;
     case HX_BF16:
       moe_combine_kernel<BF16><<<grid, block, 0, s>>>((u16*)out, (const u16*)y, row_of, weights, (const u16*)shared, shared_gate,
-                                                      gate_stride, top, width);
+                                                      gate_stride, top, width, (const u16*)identity, identity_stride);
       break;
     default: return HX_ERR_DTYPE;
   }

@@ -39,27 +39,32 @@ __device__ __forceinline__ float act_apply(float x, int act) {
 __device__ __forceinline__ float softplus(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
 
 // ------------------------------------------------------------------------------------------------ causal convolution
+// (y2, w2, bias2: a second convolution of the same inputs, or NULL; skip: the input itself is added to every result)
 template <typename A>
 __global__ __launch_bounds__(256) void causal_conv_kernel(typename A::storage* y, int64_t y_stride, const typename A::storage* u,
                                                           int64_t u_stride, const float* w, const float* bias, int act,
                                                           const float* state, int64_t slot_stride, const int32_t* slots,
                                                           const int32_t* tok_seq, const int32_t* q_cu, const int32_t* positions,
-                                                          int C, int taps) {
+                                                          int C, int taps, typename A::storage* y2, int64_t y2_stride,
+                                                          const float* w2, const float* bias2, int skip) {
   const int64_t t = blockIdx.x;
   const int seq = tok_seq[t];
   const int64_t t0 = q_cu[seq];
   const bool fresh = positions[t0] == 0;
   const float* st = state + (int64_t)slots[seq] * slot_stride;
   for (int c = blockIdx.y * 256 + threadIdx.x; c < C; c += gridDim.y * 256) {
-    float acc = bias ? bias[c] : 0.f;
+    float acc = bias ? bias[c] : 0.f, acc2 = bias2 ? bias2[c] : 0.f, x = 0.f;
     for (int j = 0; j < taps; ++j) {
       const int64_t src = t - (taps - 1) + j;
-      float x = 0.f;
+      x = 0.f;
       if (src >= t0) x = A::to_float(u[src * u_stride + c]);
       else if (!fresh) x = st[(int64_t)((taps - 1) - (int)(t0 - src)) * C + c];
       acc += w[(int64_t)c * taps + j] * x;
+      if (y2) acc2 += w2[(int64_t)c * taps + j] * x;
     }
-    y[t * y_stride + c] = A::from_float(act_apply<A>(acc, act));
+    const float own = skip ? x : 0.f;      // (the last tap's input is the token's own)
+    y[t * y_stride + c] = A::from_float(act_apply<A>(acc, act) + own);
+    if (y2) y2[t * y2_stride + c] = A::from_float(act_apply<A>(acc2, act) + own);
   }
 }
 
@@ -91,26 +96,30 @@ template <> struct Chan<BF16, 2> {
   }
 };
 
-template <typename A, int MT, int NC>
+template <typename A, int MT, int NC, bool TWO>
 __global__ __launch_bounds__(256) void causal_conv_tile_kernel(typename A::storage* y, int64_t y_stride, const typename A::storage* u,
                                                                int64_t u_stride, const float* w, const float* bias, int act,
                                                                const float* state, int64_t slot_stride, const int32_t* slots,
                                                                const int32_t* tok_seq, const int32_t* q_cu, const int32_t* positions,
-                                                               int64_t T, int C, int taps) {
+                                                               int64_t T, int C, int taps, typename A::storage* y2, int64_t y2_stride,
+                                                               const float* w2, const float* bias2, int skip) {
   const int c = NC * (blockIdx.y * 256 + threadIdx.x);
   if (c >= C) return;
   const int64_t tile0 = (int64_t)blockIdx.x * kConvTile;
   const int64_t tile1 = tile0 + kConvTile < T ? tile0 + kConvTile : T;
   const int keep = taps - 1;
   float wt[NC][MT], hist[NC][MT], b[NC];    // wt[.][j]: the weight of the input j tokens back; hist[.][j]: the input j + 1 tokens back
+  float wt2[TWO ? NC : 1][TWO ? MT : 1], b2[TWO ? NC : 1];      // the second convolution's
 #pragma unroll
   for (int n = 0; n < NC; ++n) {
 #pragma unroll
     for (int j = 0; j < MT; ++j) {
       wt[n][j] = j < taps ? w[(int64_t)(c + n) * taps + (taps - 1 - j)] : 0.f;
+      if constexpr (TWO) wt2[n][j] = j < taps ? w2[(int64_t)(c + n) * taps + (taps - 1 - j)] : 0.f;
       hist[n][j] = 0.f;
     }
     b[n] = bias ? bias[c + n] : 0.f;
+    if constexpr (TWO) b2[n] = bias2 ? bias2[c + n] : 0.f;
   }
   // the tile's sequence ids and inputs are requested at once, before anything waits for them: a portion starts where
   // the id changes, and only there (and at the tile's first token) is the history taken afresh
@@ -149,7 +158,7 @@ __global__ __launch_bounds__(256) void causal_conv_tile_kernel(typename A::stora
         for (int n = 0; n < NC; ++n) hist[n][j] = x[n];
       }
     }
-    float x[NC], o[NC];
+    float x[NC], o[NC], o2[NC];
 #pragma unroll
     for (int n = 0; n < NC; ++n) x[n] = xs[i][n];
 #pragma unroll
@@ -157,12 +166,20 @@ __global__ __launch_bounds__(256) void causal_conv_tile_kernel(typename A::stora
       float acc = b[n] + wt[n][0] * x[n];
 #pragma unroll
       for (int j = 0; j < MT - 1; ++j) acc += wt[n][j + 1] * hist[n][j];
-      o[n] = act_apply<A>(acc, act);
+      const float own = skip ? x[n] : 0.f;
+      o[n] = act_apply<A>(acc, act) + own;
+      if constexpr (TWO) {
+        float acc2 = b2[n] + wt2[n][0] * x[n];
+#pragma unroll
+        for (int j = 0; j < MT - 1; ++j) acc2 += wt2[n][j + 1] * hist[n][j];
+        o2[n] = act_apply<A>(acc2, act) + own;
+      }
 #pragma unroll
       for (int j = MT - 2; j > 0; --j) hist[n][j] = hist[n][j - 1];
       hist[n][0] = x[n];
     }
     Chan<A, NC>::store(y + t * y_stride + c, o);
+    if constexpr (TWO) Chan<A, NC>::store(y2 + t * y2_stride + c, o2);
     }
   }
 }
@@ -621,34 +638,42 @@ inline unsigned flat_blocks(int64_t total) {
     default: return HX_ERR_DTYPE;                \
   }
 
-extern "C" int hxm_causal_conv(void* y, int64_t y_stride, const void* u, int64_t u_stride, const float* w, const float* bias, int act,
-                               float* state, int64_t slot_stride, const int32_t* slots, const int32_t* tok_seq, const int32_t* q_cu,
-                               const int32_t* positions, int64_t n_tokens, int32_t n_seq, int32_t channels, int32_t taps, int dtype,
-                               void* stream) {
+static int causal_conv_launch(void* y, int64_t y_stride, const void* u, int64_t u_stride, const float* w, const float* bias, int act,
+                              float* state, int64_t slot_stride, const int32_t* slots, const int32_t* tok_seq, const int32_t* q_cu,
+                              const int32_t* positions, int64_t n_tokens, int32_t n_seq, int32_t channels, int32_t taps, int dtype,
+                              void* stream, void* y2, int64_t y2_stride, const float* w2, const float* bias2, int skip) {
   if (n_tokens < 0 || n_seq < 0 || channels < 1 || taps < 1) return HX_ERR_SHAPE;
   if (n_tokens == 0 || n_seq == 0) return HX_OK;
-  if (!y || !u || !w || !state || !slots || !tok_seq || !q_cu || !positions) return HX_ERR_NULL;
-  if (y_stride < channels || u_stride < channels) return HX_ERR_STRIDE;
+  if (!y || !u || !w || !state || !slots || !tok_seq || !q_cu || !positions || (y2 && !w2)) return HX_ERR_NULL;
+  if (y_stride < channels || u_stride < channels || (y2 && y2_stride < channels)) return HX_ERR_STRIDE;
   hipStream_t s = (hipStream_t)stream;
   const unsigned cb = (unsigned)((channels + 255) / 256);
   const dim3 grid((unsigned)n_tokens, cb < 64 ? cb : 64), sgrid((unsigned)n_seq, cb < 64 ? cb : 64), block(256);
   const uintptr_t pair = dtype == HX_F32 ? 8 : 4;
-  const bool two = channels % 2 == 0 && y_stride % 2 == 0 && u_stride % 2 == 0 && (uintptr_t)y % pair == 0 && (uintptr_t)u % pair == 0;
+  const bool two = channels % 2 == 0 && y_stride % 2 == 0 && u_stride % 2 == 0 && (uintptr_t)y % pair == 0 && (uintptr_t)u % pair == 0 &&
+                   y2_stride % 2 == 0 && (uintptr_t)y2 % pair == 0;
   const dim3 tgrid((unsigned)((n_tokens + kConvTile - 1) / kConvTile), two ? (unsigned)((channels / 2 + 255) / 256) : cb);
   auto tile = [&](auto tag, auto mt) {
     typedef decltype(tag) A;
     constexpr int MT = decltype(mt)::value;
     typedef typename A::storage E;
-    if (two)
-      causal_conv_tile_kernel<A, MT, 2><<<tgrid, block, 0, s>>>((E*)y, y_stride, (const E*)u, u_stride, w, bias, act, state, slot_stride, slots,
-                                                                tok_seq, q_cu, positions, n_tokens, channels, taps);
-    else
-      causal_conv_tile_kernel<A, MT, 1><<<tgrid, block, 0, s>>>((E*)y, y_stride, (const E*)u, u_stride, w, bias, act, state, slot_stride, slots,
-                                                                tok_seq, q_cu, positions, n_tokens, channels, taps);
+#define HXM_CONV_TILE(NC_, TWO_)                                                                                                      \
+  causal_conv_tile_kernel<A, MT, NC_, TWO_><<<tgrid, block, 0, s>>>((E*)y, y_stride, (const E*)u, u_stride, w, bias, act, state, slot_stride, \
+                                                                    slots, tok_seq, q_cu, positions, n_tokens, channels, taps, (E*)y2,   \
+                                                                    y2_stride, w2, bias2, skip)
+    if (two) {
+      if (y2) HXM_CONV_TILE(2, true);
+      else HXM_CONV_TILE(2, false);
+    } else {
+      if (y2) HXM_CONV_TILE(1, true);
+      else HXM_CONV_TILE(1, false);
+    }
+#undef HXM_CONV_TILE
   };
   typedef std::integral_constant<int, 4> Taps4;
   typedef std::integral_constant<int, 8> Taps8;
-  if (taps <= 8 && n_tokens >= kConvTile) {
+  // (a batch of few tokens — decode steps — has nothing to keep in registers from one token to the next: a thread a token and channel)
+  if (taps <= 8 && n_tokens >= 8 * kConvTile) {
     if (taps <= 4) {
       HXM_BY_DTYPE(dtype, (tile(F32{}, Taps4{})), (tile(BF16{}, Taps4{})))
     } else {
@@ -657,9 +682,11 @@ extern "C" int hxm_causal_conv(void* y, int64_t y_stride, const void* u, int64_t
   } else {
     HXM_BY_DTYPE(dtype,
                  (causal_conv_kernel<F32><<<grid, block, 0, s>>>((float*)y, y_stride, (const float*)u, u_stride, w, bias, act, state, slot_stride,
-                                                                 slots, tok_seq, q_cu, positions, channels, taps)),
+                                                                 slots, tok_seq, q_cu, positions, channels, taps, (float*)y2, y2_stride, w2,
+                                                                 bias2, skip)),
                  (causal_conv_kernel<BF16><<<grid, block, 0, s>>>((u16*)y, y_stride, (const u16*)u, u_stride, w, bias, act, state, slot_stride,
-                                                                  slots, tok_seq, q_cu, positions, channels, taps)))
+                                                                  slots, tok_seq, q_cu, positions, channels, taps, (u16*)y2, y2_stride, w2,
+                                                                  bias2, skip)))
   }
   int rc = hxm::check_launch();
   if (rc != HX_OK || taps == 1) return rc;
@@ -669,6 +696,23 @@ extern "C" int hxm_causal_conv(void* y, int64_t y_stride, const void* u, int64_t
                (causal_conv_state_kernel<BF16><<<sgrid, block, 0, s>>>((const u16*)u, u_stride, state, slot_stride, slots, q_cu, positions,
                                                                        channels, taps)))
   return hxm::check_launch();
+}
+
+extern "C" int hxm_causal_conv(void* y, int64_t y_stride, const void* u, int64_t u_stride, const float* w, const float* bias, int act,
+                               float* state, int64_t slot_stride, const int32_t* slots, const int32_t* tok_seq, const int32_t* q_cu,
+                               const int32_t* positions, int64_t n_tokens, int32_t n_seq, int32_t channels, int32_t taps, int dtype,
+                               void* stream) {
+  return causal_conv_launch(y, y_stride, u, u_stride, w, bias, act, state, slot_stride, slots, tok_seq, q_cu, positions, n_tokens, n_seq,
+                            channels, taps, dtype, stream, nullptr, 0, nullptr, nullptr, 0);
+}
+
+extern "C" int hxm_causal_conv_pair(void* y, int64_t y_stride, void* y2, int64_t y2_stride, const void* u, int64_t u_stride,
+                                    const float* w, const float* w2, const float* bias, const float* bias2, int act, int skip,
+                                    float* state, int64_t slot_stride, const int32_t* slots, const int32_t* tok_seq,
+                                    const int32_t* q_cu, const int32_t* positions, int64_t n_tokens, int32_t n_seq, int32_t channels,
+                                    int32_t taps, int dtype, void* stream) {
+  return causal_conv_launch(y, y_stride, u, u_stride, w, bias, act, state, slot_stride, slots, tok_seq, q_cu, positions, n_tokens, n_seq,
+                            channels, taps, dtype, stream, y2, y2_stride, w2, bias2, skip);
 }
 
 extern "C" int hxm_token_shift_mix(void* out, const void* h, int64_t h_stride, const float* mu, int32_t n_mix, float* state,

@@ -41,33 +41,12 @@ from hydrainfer_amd._C.kernel.depth_ops import depth_norm
 from hydrainfer_amd._C.kernel.seq_mix import (causal_conv, clamped_glu, decay_exp, gated_group_norm, head_gates,
                                               head_norm_rope_cache, state_scan, token_shift_mix, unary, unit_norm)
 from hydrainfer_amd._C.kernel.stream_ops import SequenceState, stream_embed
+from hydrainfer_amd.layer.rotary_spec import RotarySpec
 
 ARCHITECTURE = "Fasanex"
 GLU_ALPHA = 1.702             # the feed-forward's gate: g sigmoid(GLU_ALPHA g)
 UNIT_NORM_EPS = 1e-6          # delta rule: q, k / sqrt(sum of squares + UNIT_NORM_EPS)
 SHIFT_MIXES = ("r", "k", "v", "g", "w")
-
-
-@dataclass
-class RotarySpec:
-    dims: int
-    base: float
-    factor: Optional[float] = None      # YaRN: None = plain frequencies
-    original: float = 0.0
-    fast: float = 32.0
-    slow: float = 1.0
-
-    def frequencies(self) -> Tuple[List[float], float]:
-        """(angle per position of every pair [dims / 2], factor on cos and sin).  With YaRN the pairs that turn fast keep
-        their frequency, the slow ones are divided by `factor`, with a linear ramp between."""
-        f = [self.base ** (-2.0 * i / self.dims) for i in range(self.dims // 2)]
-        if not self.factor:
-            return f, 1.0
-        turn = lambda t: self.dims * math.log(self.original / (2.0 * math.pi * t)) / (2.0 * math.log(self.base))
-        lo = max(math.floor(turn(self.fast)), 0)
-        hi = min(math.ceil(turn(self.slow)), self.dims - 1)
-        ramp = [min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0) for i in range(self.dims // 2)]
-        return [fi / self.factor * r + fi * (1.0 - r) for fi, r in zip(f, ramp)], 0.1 * math.log(self.factor) + 1.0
 
 
 @dataclass

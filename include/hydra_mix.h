@@ -10,7 +10,10 @@
  * and, for mixers that keep per-sequence state beside the cache: short causal convolutions, token shift with several
  * mixes, per-head RMS norm + rotary positions + cache append, decays / step sizes / write strengths of a recurrence, a scan
  * over a matrix state per head in three forms (decayed sum, read-before-write with a bonus, delta rule), the gate / group
- * norm that finishes a mixer, and a clamped gated feed-forward activation.
+ * norm that finishes a mixer, and a clamped gated feed-forward activation; and, for attention with sinks: a learned extra
+ * term in the softmax's denominator and a temperature per head (both attention kernels), rotary positions over parts of a
+ * token's row in either pair layout with values that turn too (hxm_rotary_parts), two short convolutions of one input
+ * added to it, identity experts and un-renormalised router weights.
  *
  * Same conventions as hydra_hip.h: raw device pointers, sizes and strides in ELEMENTS, a hipStream_t passed as void*,
  * asynchronous launches, no allocation, 0 or a negative hx_status (hydra_hip.h) as the result.  `dtype` is the hx_dtype
@@ -28,7 +31,7 @@
 extern "C" {
 #endif
 
-#define HXM_ABI_VERSION 3
+#define HXM_ABI_VERSION 4
 #define HXM_MAX_STREAMS 16
 #define HXM_MAX_LATENT 1024     /* widest latent row the attention kernels hold in registers (the MFMA tile form: 512) */
 
@@ -107,6 +110,8 @@ typedef struct hxm_latent_attn_args {
   int32_t n_splits;          /* from hxm_latent_attention_plan; > 1: the key range of a row tile is dealt to n_splits waves */
   float* ws_o;               /* n_splits > 1: the plan's workspace, ws_floats floats; ws_ml = where its (max, sum) pairs go */
   float* ws_ml;
+  const float* sinks;        /* [n_heads] or NULL: the softmax's denominator of head h holds one more term exp(sinks[h]), which
+                                has no key and no value (an attention sink); it is not scaled */
 } hxm_latent_attn_args;
 
 /* How a launch with these arguments would be laid out: n_splits (1: no workspace) and the floats of workspace it needs
@@ -130,14 +135,24 @@ int hxm_embed_positions(float* out, const void* table, const void* pos_table, co
 
 /* One row kernel for every place where a residual meets a norm.  LN(u) = (u - mean(u)) / sqrt(var(u) + eps), var the mean
  * squared deviation; with rms != 0: LN(u) = u / sqrt(mean(u^2) + eps).  For output row i (input row r = rows ? rows[i] : i):
- *   x = x_in[r]
- *   if y:         x += mult * LN(y[r]) * post_w                      (a sublayer's result enters the residual)
+ *   x = x_in ? x_in[r] : 0
+ *   if y:         x += mult * N(y[r]) * post_w                       (a sublayer's result enters the residual; N by post_norm:
+ *                                                                     LN as above, the layer norm, the RMS norm, or y as it is —
+ *                                                                     then post_w may be NULL: ones)
+ *   if y2:        x += y2[r]                                         (a second sublayer that read the same input)
+ *   if bias:      x += bias                                          (a float vector of `width`)
  *   if level_out: level_out[r] = x                                   (the layer's own result joins the stack of levels)
  *   if depth_w:   x = sum_{j < n_levels} depth_w[j] * levels[j][r]   (levels[j] = levels + j * level_stride; may include
  *                                                                     the level just written)
  *   if x_out:     x_out[i] = x
  *   if next_w:    h_out[i] = LN(x) * next_w                          (dtype; the next sublayer's input)
- * x_in, level_out, levels, x_out: float rows of `width` (contiguous).  y: dtype, row stride y_stride. */
+ *   else if h_out: h_out[i] = x                                      (dtype; the residual as a matrix product's operand)
+ * x_in, level_out, levels, x_out: float rows of `width` (contiguous).  y, y2: dtype, row strides y_stride, y2_stride; h_out:
+ * dtype, row stride h_stride (so that it may be a column range of a wider matrix). */
+#define HXM_POST_SAME 0     /* y is normed like everything else in the call (rms) */
+#define HXM_POST_LAYER 1    /* layer norm */
+#define HXM_POST_RMS 2      /* RMS norm */
+#define HXM_POST_PLAIN 3    /* no norm */
 typedef struct hxm_depth_norm_args {
   const float* x_in;
   const void* y;
@@ -152,6 +167,10 @@ typedef struct hxm_depth_norm_args {
   int64_t y_stride, level_stride, n_out, width;
   int32_t n_levels, rms, dtype;
   float mult, eps;
+  const void* y2;
+  const float* bias;
+  int64_t y2_stride, h_stride;
+  int32_t post_norm;         /* HXM_POST_* */
 } hxm_depth_norm_args;
 int hxm_depth_norm(const hxm_depth_norm_args* args, void* stream);
 
@@ -169,10 +188,12 @@ int hxm_relu_squared(void* out, int64_t out_stride, const void* z, int64_t z_str
  * ------------------------------------------------------------------------------------------------------------------ */
 
 /* s = softmax(logits[t, 0 : n_experts]); the `top` experts with the largest s + choice_bias (NULL: s; ties: the lower
- * expert) are chosen; weights[t, k] = s[chosen k] / (sum of the chosen s + 1e-20) * scale.  logits: float, row stride
- * logit_stride.  weights: float [n_tokens, top], experts: int32 [n_tokens, top], in order of decreasing choice score. */
+ * expert) are chosen; weights[t, k] = s[chosen k] / (sum of the chosen s + 1e-20) * scale, or with renorm == 0 the chosen
+ * scores themselves, s[chosen k] * scale.  logits: float, row stride logit_stride.  weights: float [n_tokens, top],
+ * experts: int32 [n_tokens, top], in order of decreasing choice score. */
 int hxm_route_softmax_topk(const float* logits, int64_t logit_stride, const float* choice_bias, int64_t n_tokens,
-                           int32_t n_experts, int32_t top, float scale, float* weights, int32_t* experts, void* stream);
+                           int32_t n_experts, int32_t top, float scale, int32_t renorm, float* weights, int32_t* experts,
+                           void* stream);
 
 /* Expert-major order of the n = n_tokens * top (token, choice) pairs: seg[e] .. seg[e + 1] are the rows of expert e
  * (int32 [n_experts + 1]); row_of[t * top + k] = the row of pair (t, k); src[row] = t.  One launch of one workgroup. */
@@ -186,10 +207,12 @@ int hxm_grouped_linear(void* y, const void* x, int64_t x_stride, const int32_t* 
                        int64_t max_rows, int32_t n_experts, int64_t n_dim, int64_t k_dim, int32_t act, int dtype, void* stream);
 
 /* out[t, :] = sum_k weights[t, k] * y[row_of[t * top + k], :] + (shared ? sigmoid(shared_gate[t * gate_stride]) * shared[t, :] : 0).
- * y, shared, out: dtype rows of `width`; weights, shared_gate: float. */
+ * A choice whose row_of is negative (an expert beyond the n_experts hxm_moe_plan was called with) adds nothing — or, with
+ * `identity` (dtype rows of `width`, row stride identity_stride: the experts' input), weights[t, k] * identity[t, :]: experts
+ * without tensors that hand their input on.  y, shared, out: dtype rows of `width`; weights, shared_gate: float. */
 int hxm_moe_combine(void* out, const void* y, const int32_t* row_of, const float* weights, const void* shared,
-                    const float* shared_gate, int64_t gate_stride, int64_t n_tokens, int32_t top, int64_t width, int dtype,
-                    void* stream);
+                    const float* shared_gate, int64_t gate_stride, const void* identity, int64_t identity_stride,
+                    int64_t n_tokens, int32_t top, int64_t width, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------------------------------
  * Gated linear recurrence with a matrix state per head (HGRN2): f = low + (1 - low) * sigmoid(f_pre + f_bias) per head and
@@ -251,6 +274,9 @@ typedef struct hxm_biased_attn_args {
   float* ws_o;               /* n_splits > 1: n_seq * kv_heads * ceil(max_q_len * heads / kv_heads / 16) * n_splits * 16 * ceil16(vdim) floats */
   float* ws_ml;              /* n_splits > 1: ... * n_splits * 32 floats */
   float softcap;             /* > 0: q . k * scale becomes softcap * tanh(q . k * scale / softcap) before the bias; 0: none */
+  const float* head_scale;   /* [n_heads] or NULL: head h's scores are q . k * scale * head_scale[h] (a temperature per head) */
+  const float* sinks;        /* [n_heads] or NULL: the softmax's denominator of head h holds one more term exp(sinks[h]), which
+                                has no key and no value (an attention sink); it is not scaled */
 } hxm_biased_attn_args;
 
 /* Softmax attention of every query over the keys of its own sequence that its mask lets it see (scores and weights in
@@ -279,6 +305,16 @@ int hxm_causal_conv(void* y, int64_t y_stride, const void* u, int64_t u_stride, 
                     float* state, int64_t slot_stride, const int32_t* slots, const int32_t* tok_seq, const int32_t* q_cu,
                     const int32_t* positions, int64_t n_tokens, int32_t n_seq, int32_t channels, int32_t taps, int dtype,
                     void* stream);
+
+/* Up to two convolutions of the same inputs in one pass (an input is read once, and the slot brought up to date once):
+ * y = act(conv_w(u) + bias) + (skip ? u : 0), and, when y2 is given, y2 = act(conv_w2(u) + bias2) + (skip ? u : 0).  A mixer
+ * and a feed-forward that read the same normed input, each through a short convolution of its own added to that input,
+ * are one call with skip = 1. */
+int hxm_causal_conv_pair(void* y, int64_t y_stride, void* y2, int64_t y2_stride, const void* u, int64_t u_stride, const float* w,
+                         const float* w2, const float* bias, const float* bias2, int act, int skip, float* state,
+                         int64_t slot_stride, const int32_t* slots, const int32_t* tok_seq, const int32_t* q_cu,
+                         const int32_t* positions, int64_t n_tokens, int32_t n_seq, int32_t channels, int32_t taps, int dtype,
+                         void* stream);
 
 /* out[m, t, :] = h[t] + (h[t - 1] - h[t]) * mu[m] for m < n_mix, h[t - 1] of the same sequence (zeros before position 0;
  * across portions through the slot's `width` floats, left holding the portion's last h).  h: dtype [n_tokens, width]
@@ -333,6 +369,40 @@ typedef struct hxm_head_rope_args {
 /* Per-head RMS norm (plain weight) of queries and keys, rotary positions on the first rot_dims channels of every head
  * (angles, cos and sin in float), keys and values appended to the paged cache. */
 int hxm_head_norm_rope_cache(const hxm_head_rope_args* args, void* stream);
+
+#define HXM_ROT_HALVES 0        /* channel i turns with channel i + dims / 2 */
+#define HXM_ROT_INTERLEAVED 1   /* channel 2 i turns with channel 2 i + 1 */
+#define HXM_GATE_PER_HEAD 1     /* gate: one number per head, rows of `heads` */
+#define HXM_GATE_PER_ELEMENT 2  /* gate: one number per element, rows of heads * size */
+#define HXM_ROT_MAX_PARTS 3
+
+typedef struct hxm_rotary_part {
+  const void* src;           /* dtype rows: head h of token t at src + t * src_stride + h * src_head_stride, `size` elements */
+  void* dst;                 /* dtype rows (dst_stride a token), or the paged cache when to_cache: the token's row is at
+                                dst + block * cache_block_stride + row * dst_stride, (block, row) from its slot id */
+  const double* inv_freq;    /* [rot_dims / 2]: pair i turns by position * inv_freq[i]; NULL: nothing turns (a copy, or a gate) */
+  const void* gate;          /* dtype, optional: the result is multiplied by sigmoid(gate), rows of gate_stride a token */
+  int64_t src_stride, src_head_stride, dst_stride, dst_head_stride, cache_block_stride, gate_stride;
+  int32_t heads, size;       /* heads of the part, elements of a head */
+  int32_t rot_off, rot_dims; /* channels rot_off .. rot_off + rot_dims - 1 of every head turn, the others are copied */
+  int32_t layout;            /* HXM_ROT_* */
+  int32_t to_cache;
+  int32_t gate_kind;         /* HXM_GATE_* */
+  float mag;                 /* cos and sin are multiplied by mag */
+  float sign;                /* 1: turn by + position; -1: turn back */
+} hxm_rotary_part;
+
+typedef struct hxm_rotary_args {
+  hxm_rotary_part parts[HXM_ROT_MAX_PARTS];
+  const int32_t* positions;  /* [n_tokens] */
+  const int32_t* slot_ids;   /* [n_tokens] cache slot (block * block_size + row) of every token; < 0: the token's cache parts are skipped */
+  int64_t n_tokens;
+  int32_t n_parts, block_size, dtype;
+} hxm_rotary_args;
+
+/* Rotary positions over up to three groups of heads of every token in one launch (angles and their cos / sin from the
+ * position in double); see hxm_rotary_part.  A part may be turned in place (dst == src with equal strides). */
+int hxm_rotary_parts(const hxm_rotary_args* args, void* stream);
 
 #define HXM_SCAN_DECAY 0      /* S <- a S + k (s v)^T;  o = S^T q */
 #define HXM_SCAN_BONUS 1      /* o = (S + diag(u) k v^T)^T q;  then S <- a S + k v^T */
