@@ -69,7 +69,17 @@ def _load_fasanex(model_path: str, dtype, device, **_):
     return TextLanguageModel(model), None
 
 
+def _load_pemalorn(model_path: str, dtype, device, **_):
+    from hydrainfer_amd.model.llava import TextLanguageModel
+    from hydrainfer_amd.model.loader import scan_safetensors
+    from hydrainfer_amd.model.pemalorn import PemalornForCausalLM, read_shape
+    shape = read_shape(model_path)
+    model = PemalornForCausalLM.from_state_dict(shape, scan_safetensors(model_path, ("",)), dtype, device)
+    return TextLanguageModel(model), None
+
+
 register("LlavaForConditionalGeneration", _load_llava)
 register("Tetepel", _load_tetepel)
 register("Kezolix", _load_kezolix)
 register("Fasanex", _load_fasanex)
+register("Pemalorn", _load_pemalorn)
