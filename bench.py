@@ -79,7 +79,7 @@ def parse():
     p.add_argument("--no-ragged", action="store_true", help="skip whole_step_ragged (the decode step on ragged batches)")
     p.add_argument("--no-null-step", action="store_true",
                    help="skip whole_step.null_step (the launch structure's ceiling: the step with math-free stand-in launches)")
-    p.add_argument("--design", default=None, choices=["tetepel", "kezolix", "fasanex"],
+    p.add_argument("--design", default=None, choices=["tetepel", "kezolix", "fasanex", "pemalorn"],
                    help="instead of the default workload: prefill / decode throughput of this model design at layer sizes of a "
                         "real model (random weights) beside the Llama decoder at equal size, and its kernels against the Llama "
                         "path's like kernels as fractions of their rooflines (hydrainfer_amd/utils/design_bench.py); 1 GPU")
@@ -1493,7 +1493,7 @@ def leg_13b_child(args):
 
 
 def design_leg(args):
-    """`--design tetepel|kezolix|fasanex`: one JSON line — the design's throughput and kernel table beside the Llama decoder's."""
+    """`--design tetepel|kezolix|fasanex|pemalorn`: one JSON line — the design's throughput and kernel table beside the Llama decoder's."""
     from hydrainfer_amd.utils import design_bench
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)

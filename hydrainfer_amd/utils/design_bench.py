@@ -1,4 +1,4 @@
-"""`bench.py --design tetepel|kezolix|fasanex`: prefill and decode throughput of a model design at sizes that resemble a real
+"""`bench.py --design tetepel|kezolix|fasanex|pemalorn`: prefill and decode throughput of a model design at sizes that resemble a real
 model's layers (random weights, a few layers), beside the Llama decoder at equal width / feed-forward / heads (Fasanex:
 also beside Kezolix, the closest design), and a table of the design's own kernels against the like kernels of the models
 beside it, each as a fraction of its roofline (HBM bytes or MFMA flops, algorithmic counts).  All models run their eager
@@ -61,6 +61,33 @@ def _fasanex(size: dict, dtype, dev):
     return FasanexForCausalLM.random_init(shape, dtype, dev, seed=0)
 
 
+def _pemalorn_sizes(size: dict) -> dict:
+    """Attention as wide as the Llama decoder's, a quarter of the heads carrying keys, half of every head turning; latent
+    attention with the size's latents, 64 rotated channels beside them (a cached row of at most 512 columns keeps the
+    matrix-core form) and a window of 512; 16 experts of a quarter of the dense inner size, four a token, two identity
+    experts; four taps; 64 channels of per-layer token input."""
+    H, D = size["heads"], size["dim"]
+    return dict(H=H, G=H // 4, D=D, V=D, rot=D // 2, R=64, C=min(size["kv_rank"], 512 - 64), Q=size["q_rank"], window=512,
+                E=16, I=2, top=4, eff=size["ff"] // 4 // 32 * 32, taps=4, side=64)
+
+
+def _pemalorn(size: dict, dtype, dev):
+    """Four layers — attention, latent attention, attention, latent attention, a mixture of experts beside each — the two
+    in the middle entered through the loop's input product (one pass)."""
+    from hydrainfer_amd.layer.rotary_spec import RotarySpec
+    from hydrainfer_amd.model.pemalorn import ExpertsSpec, MixerSpec, PemalornForCausalLM, PemalornLayer, PemalornShape
+    z = _pemalorn_sizes(size)
+    att = MixerSpec("attention", heads=z["H"], dim=z["D"], vdim=z["V"], scale=1.0 / math.sqrt(z["D"]), kv_heads=z["G"],
+                    rot=RotarySpec(z["rot"], 10000.0))
+    lat = MixerSpec("latent_attention", heads=z["H"], dim=z["D"], vdim=z["V"], scale=1.0 / math.sqrt(z["D"] + z["R"]), kv_rank=z["C"],
+                    q_rank=z["Q"], rot_dim=z["R"], window=z["window"], rot=RotarySpec(z["R"], 10000.0, 4.0, 4096.0, 32.0, 1.0))
+    moe = ExpertsSpec(z["E"], z["I"], z["top"], z["eff"])
+    layers = [PemalornLayer(m, moe) for m in (att, lat, att, lat)][:size["layers"]]
+    shape = PemalornShape(VOCAB, size["width"], layers, norm_eps=1e-5, taps=z["taps"], side_dim=z["side"], loop_start=1,
+                          loop_stop=min(3, len(layers)), loop_times=1, has_loop=len(layers) > 1)
+    return PemalornForCausalLM.random_init(shape, dtype, dev, seed=0)
+
+
 def _llama(size: dict, dtype, dev):
     from hydrainfer_amd.model.llama import LlamaForCausalLM, LlamaShape
     shape = LlamaShape(size["width"], size["ff"], size["layers"], size["heads"], size["heads"], size["dim"], VOCAB)
@@ -98,7 +125,7 @@ def _batch(model, n_seqs: int, q_len: int, kv_len: int, dtype, dev):
 
 
 # the models a design's throughput is set beside: the closest existing one first
-BESIDE = {"fasanex": ("kezolix", "llama")}
+BESIDE = {"fasanex": ("kezolix", "llama"), "pemalorn": ("kezolix", "tetepel", "llama")}
 
 
 def _time_eager(fn: Callable, dev, reps: int = 5, warm: int = 2) -> float:
@@ -148,7 +175,7 @@ def _row(name, us, nbytes=None, flops=None):
 def throughput(size_name: str, dtype, dev, prefill=(4, 1024), decode=(32, 1024), design: str = "tetepel") -> dict:
     size = SIZES[size_name]
     out = {}
-    makers = {"tetepel": _tetepel, "kezolix": _kezolix, "fasanex": _fasanex, "llama": _llama}
+    makers = {"tetepel": _tetepel, "kezolix": _kezolix, "fasanex": _fasanex, "pemalorn": _pemalorn, "llama": _llama}
     beside = BESIDE.get(design, ("llama",))
     for name, make in [(n, makers[n]) for n in (design,) + beside]:
         model = make(size, dtype, dev)
@@ -535,11 +562,141 @@ def fasanex_kernel_table(size_name: str, dtype, dev, T: int = 4096, n_seqs: int 
     return rows
 
 
+def pemalorn_kernel_table(size_name: str, dtype, dev, T: int = 4096, n_seqs: int = 4, B: int = 32, ctx: int = 2048) -> dict:
+    """Every kernel of the Pemalorn design at a prefill batch of T tokens (n_seqs portions) — the attentions also at a decode
+    batch of B sequences — and beside them the tables of the two closest designs at the same sizes: Kezolix (grouped-query
+    attention of the same kernel family, experts, the same residual kernel) and Tetepel (latent attention)."""
+    from hydrainfer_amd._C.kernel import biased_attn as ba, depth_ops as do, moe_mix as mm
+    from hydrainfer_amd._C.kernel.latent_attn import latent_attention, latent_norm_cache
+    from hydrainfer_amd._C.kernel.rotary import RotaryPart, rotary_parts
+    from hydrainfer_amd._C.kernel.seq_mix import causal_conv_pair, clamped_glu, gated_group_norm
+    from hydrainfer_amd._C.kernel.stream_ops import SequenceState, gelu_tanh_and_mul
+    from hydrainfer_amd.layer.rotary_spec import RotarySpec
+    sz = SIZES[size_name]
+    z = _pemalorn_sizes(sz)
+    W, H, G, D, V, C, R, Q = sz["width"], z["H"], z["G"], z["D"], z["V"], z["C"], z["R"], z["Q"]
+    E, I, top, eff, taps, side, win = z["E"], z["I"], z["top"], z["eff"], z["taps"], z["side"], z["window"]
+    e = 2
+    rnd = lambda *s: torch.randn(s, device=dev).to(dtype)
+    f32 = lambda *s: torch.randn(s, device=dev)
+    f64 = lambda v: torch.tensor(v, dtype=torch.float64, device=dev)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev) if not torch.is_tensor(v) else v.to(torch.int32).to(dev)
+    rows: Dict[str, List[dict]] = {"pemalorn": []}
+    add = lambda *a, **k: rows["pemalorn"].append(_row(*a, **k))
+    q_len = T // n_seqs
+    q_cu = i32(list(range(0, T + 1, q_len)))
+    pos = torch.arange(q_len, dtype=torch.int32, device=dev).repeat(n_seqs)
+    tok_seq = torch.arange(n_seqs, dtype=torch.int32, device=dev).repeat_interleave(q_len)
+    posd, qcud, seq_ids = i32([ctx - 1] * B), i32(list(range(B + 1))), i32(list(range(B)))
+    # residual
+    x, y, y2, w1, w2 = f32(T, W), rnd(T, W), rnd(T, W), f32(W), f32(W)
+    xo, xb = torch.empty_like(x), torch.empty((T, W), dtype=dtype, device=dev)
+    us = _time_graph(lambda: do.depth_norm(x, dtype, 1e-5, y=y, post_norm="plain", y2=y2, x_out=xo, cast_out=xb), dev)
+    add("depth_norm: mixer and experts into the residual + operand copy", us, T * W * (8 + 3 * e))
+    us = _time_graph(lambda: do.depth_norm(x, dtype, 1e-5, y=y, post_w=w1, post_norm="rms", x_out=xo, next_w=w2), dev)
+    add("depth_norm: RMS norm of the token input into the residual + next layer norm", us, T * W * (8 + 2 * e))
+    # input convolutions
+    h, cw1, cw2 = rnd(T, W), f32(W, taps), f32(W, taps)
+    state = torch.zeros((max(n_seqs, B), 1, (taps - 1) * W), device=dev)
+    seq = SequenceState(state, i32(list(range(n_seqs))), tok_seq)
+    us = _time_graph(lambda: causal_conv_pair(h, cw1, cw2, seq, 0, q_cu, pos), dev)
+    add(f"causal_conv_pair: two convolutions of {taps} taps added to their input", us, 3 * T * W * e)
+    # attention mixer
+    hs = max(D, V)
+    nb, nbd = (q_len + 15) // 16, (ctx + 15) // 16
+    table, cu_b = i32(torch.randperm(n_seqs * nb)), i32(list(range(0, n_seqs * nb + 1, nb)))
+    slots = i32([int(table[s * nb + p // 16]) * 16 + p % 16 for s in range(n_seqs) for p in range(q_len)])
+    kp, vp = rnd(n_seqs * nb, 16, 1, G * hs), rnd(n_seqs * nb, 16, 1, G * hs)
+    proj = rnd(T, (H + G) * D + G * V + H)
+    fq = f64(RotarySpec(z["rot"], 10000.0).frequencies()[0])
+    fv = f64([10000.0 ** (-2.0 * j / V) for j in range(V // 2)])
+    at_k, at_v, at_g = H * D, (H + G) * D, (H + G) * D + G * V
+    pre = lambda: rotary_parts([RotaryPart(proj[:, :at_k], H, D, fq), RotaryPart(proj[:, at_k:at_v], G, D, fq, cache=kp, cache_head_stride=hs),
+                                RotaryPart(proj[:, at_v:at_g], G, V, fv, cache=vp, cache_head_stride=hs)], pos, slots)
+    us = _time_graph(pre, dev)
+    add("rotary_parts: q, k and turning values of a token, k and v to the cache", us, 2 * T * ((H + G) * D + G * V) * e)
+    heads = lambda c: c.as_strided((c.shape[0], c.shape[1], G, hs), (c.stride(0), c.stride(1), hs, 1))
+    q, temp, sink = rnd(T, H, D), 1 + 0.1 * f32(H), f32(H)
+    seen = n_seqs * sum(i + 1 for i in range(q_len))
+    us = _time_graph(lambda: ba.biased_attention(q, heads(kp), heads(vp), V, tok_seq, pos, q_cu, table, cu_b, 1 / math.sqrt(D), None, "causal",
+                                                 0, max_q_len=q_len, kv_heads=G, max_kv_len=q_len, head_scale=temp, sinks=sink), dev, launches=2)
+    add(f"biased_attention, prefill {n_seqs} x {q_len} (causal, sinks, temperatures, head_dim {D})", us, flops=2 * H * (D + V) * seen)
+    kpd, vpd = rnd(B * nbd, 16, 1, G * hs), rnd(B * nbd, 16, 1, G * hs)
+    table_d, cu_bd = i32(torch.randperm(B * nbd)), i32(list(range(0, B * nbd + 1, nbd)))
+    qd = rnd(B, H, D)
+    us = _time_graph(lambda: ba.biased_attention(qd, heads(kpd), heads(vpd), V, seq_ids, posd, qcud, table_d, cu_bd, 1 / math.sqrt(D), None,
+                                                 "causal", 0, max_q_len=1, kv_heads=G, max_kv_len=ctx, head_scale=temp, sinks=sink), dev)
+    add(f"biased_attention, decode {B} x {ctx} keys (sinks, temperatures)", us, B * ctx * G * (D + V) * e + 2 * B * H * D * e)
+    o = rnd(T, H * V)
+    us = _time_graph(lambda: rotary_parts([RotaryPart(o, H, V, fv, back=True, gate=proj[:, at_g:], gate_kind="head")], pos), dev)
+    add("rotary_parts: heads' results turned back + gate per head", us, 2 * T * H * V * e)
+    # latent attention mixer
+    row = C + R
+    cache = rnd(n_seqs * nb, 16, 1, row)
+    lproj = rnd(T, Q + C + R + H * V)
+    qw, kw = f32(Q), f32(C)
+    us = _time_graph(lambda: latent_norm_cache(lproj, 0, Q, Q, C, qw, kw, 1e-5, slots, cache), dev)
+    add("latent_norm_cache (two norms + cache append)", us, 2 * T * (Q + C) * e)
+    ql = rnd(T, H * (D + R))
+    fl, mag = RotarySpec(R, 10000.0, 4.0, 4096.0, 32.0, 1.0).frequencies()
+    fl = f64(fl)
+    us = _time_graph(lambda: rotary_parts([RotaryPart(ql, H, D + R, fl, rot_off=D, layout="interleaved", mag=mag, dst=ql),
+                                           RotaryPart(lproj[:, Q + C:Q + C + R], 1, R, fl, layout="interleaved", mag=mag, cache=cache,
+                                                      cache_col=C)], pos, slots), dev)
+    add("rotary_parts: rotated part of the latent queries in place + shared key part to the cache", us, 2 * T * (H * (D + R) + R) * e)
+    qlat = rnd(T, H, row)
+    seen_w = n_seqs * sum(min(i + 1, win) for i in range(q_len))
+    us = _time_graph(lambda: latent_attention(qlat, cache, tok_seq, pos, q_cu, table, cu_b, 0.1, win, q_len, max_kv_len=q_len, sinks=sink), dev,
+                     launches=2)
+    add(f"latent_attention, prefill {n_seqs} x {q_len} (window {win}, sinks, cached row {row})", us, flops=4 * H * row * seen_w)
+    cache_d, qld = rnd(B * nbd, 16, 1, row), rnd(B, H, row)
+    us = _time_graph(lambda: latent_attention(qld, cache_d, seq_ids, posd, qcud, table_d, cu_bd, 0.1, win, 1, max_kv_len=ctx, sinks=sink), dev)
+    add(f"latent_attention, decode {B} x {min(ctx, win)} keys of the window", us, B * min(ctx, win) * row * e + 2 * B * H * row * e)
+    og = rnd(T, H * V)
+    us = _time_graph(lambda: gated_group_norm(og, dtype, gate=lproj[:, Q + C + R:], gate_act="sigmoid"), dev)
+    add("gated_group_norm: sigmoid gate per element on the latent attention's result", us, 3 * T * H * V * e)
+    # experts
+    logits, corr = f32(T, E + I), f32(E + I) * 0.01
+    us = _time_graph(lambda: mm.route_softmax_topk(logits, E + I, top, 1.0, corr, renorm=False), dev)
+    add(f"route_softmax_topk ({E} + {I} identity experts, top {top}, plain weights)", us, T * (E + I + 2 * top) * 4)
+    wts, idx = mm.route_softmax_topk(logits, E + I, top, 1.0, corr, renorm=False)
+    us = _time_graph(lambda: mm.moe_plan(idx, E), dev)
+    add("moe_plan (one workgroup)", us, 3 * T * top * 4)
+    seg, row_of, src = mm.moe_plan(idx, E)
+    n_rows = int(seg[-1])
+    gate_up, down = rnd(E, 2 * eff, W) / math.sqrt(W), rnd(E, W, eff) / math.sqrt(eff)
+    us = _time_graph(lambda: mm.grouped_linear(h, gate_up, seg, T * top, src=src), dev, launches=2)
+    add(f"grouped_linear gate | up ({n_rows} rows, {W} -> 2 x {eff})", us, flops=2 * n_rows * W * 2 * eff)
+    gu = mm.grouped_linear(h, gate_up, seg, T * top, src=src)
+    us = _time_graph(lambda: clamped_glu(gu[:, :eff], gu[:, eff:], 0.0, 1.0, 0.0), dev)
+    add("clamped_glu as silu(gate) * up over the experts' rows", us, 3 * T * top * eff * e)
+    act = clamped_glu(gu[:, :eff], gu[:, eff:], 0.0, 1.0, 0.0)
+    us = _time_graph(lambda: mm.grouped_linear(act, down, seg, T * top), dev, launches=2)
+    add(f"grouped_linear down ({n_rows} rows, {eff} -> {W})", us, flops=2 * n_rows * W * eff)
+    yd = mm.grouped_linear(act, down, seg, T * top)
+    us = _time_graph(lambda: mm.moe_combine(yd, row_of, wts, identity=h), dev)
+    add("moe_combine (+ identity experts)", us, T * W * (top + 2) * e)
+    # per-layer token input
+    gp, emb = rnd(T, side), rnd(T, 4 * side)
+    us = _time_graph(lambda: gelu_tanh_and_mul(gp, emb[:, side:2 * side]), dev)
+    add(f"gelu_tanh_and_mul (token input, {side} channels)", us, 3 * T * side * e)
+    del kp, vp, kpd, vpd, cache, cache_d, gate_up, down, gu, act, yd
+    torch.cuda.empty_cache()
+    kz = kezolix_kernel_table(size_name, dtype, dev, T, n_seqs, B, ctx)
+    rows["kezolix"], rows["llama"] = kz["kezolix"], kz["llama"]
+    rows["tetepel"] = kernel_table(size_name, dtype, dev, T, n_seqs, B, ctx)["tetepel"]
+    rows["workload"] = {"prefill_tokens": T, "portions": n_seqs, "decode_batch": B, "decode_keys": ctx, "size": sz, "pemalorn": z,
+                        "timing": "hipGraph of 10 (long kernels: 2) launches, mean of 3 replays, HIP events",
+                        "roofline": f"HBM {HBM_PEAK_GBS} GB/s, MFMA {MFMA_PEAK_TFLOPS} TFLOP/s dense bf16; algorithmic bytes / flops"}
+    return rows
+
+
 def run(dtype, dev, sizes=("w2048", "w4096"), design: str = "tetepel") -> dict:
     from hydrainfer_amd import _lib
     _lib.lib(); _lib.mix_lib()
     res = {"throughput": {}, "kernels": {}}
-    table = {"tetepel": kernel_table, "kezolix": kezolix_kernel_table, "fasanex": fasanex_kernel_table}[design]
+    table = {"tetepel": kernel_table, "kezolix": kezolix_kernel_table, "fasanex": fasanex_kernel_table,
+             "pemalorn": pemalorn_kernel_table}[design]
     for s in sizes:
         res["throughput"][s] = throughput(s, dtype, dev, design=design)
         res["kernels"][s] = table(s, dtype, dev)
