@@ -613,3 +613,39 @@ def test_registry_and_trace_run_command_line(tmp_path):
     _close(read(0), ra[[0, 16]], TOL32, "step 0")
     _close(read(1), ra[[17]], TOL32, "step 1")
     _close(read(2), torch.cat([ra[[20]], rb[[8]]]), TOL32, "step 2")
+
+
+def test_chat_endpoint_serves_a_checkpoint_directory(tmp_path):
+    """`python -m hydrainfer_amd.entrypoint --checkpoint DIR` in parts: registry -> node -> front end -> HTTP endpoint.  The
+    streams carry the tokens the offline engine generates for the same token ids."""
+    import asyncio
+    from types import SimpleNamespace
+    import safetensors.torch
+    from hydrainfer_amd.engine.offline import OfflineInferenceEngine, OfflineRequest
+    from hydrainfer_amd.entrypoint.__main__ import build_checkpoint_server
+    from hydrainfer_amd.entrypoint.api_protocol import parse_chat_completion_request as parse
+    from tests.test_api_server import _client_stream, _payload
+    shape = _shape("mix")
+    W = _weights(shape, seed=19)
+    (tmp_path / "config.json").write_text(json.dumps(shape.to_config()))
+    safetensors.torch.save_file({k: v.to(torch.bfloat16) for k, v in W.items()}, str(tmp_path / "model.safetensors"))
+    args = SimpleNamespace(checkpoint=str(tmp_path), max_running=4, max_tokens=128, tokenizer=None, host="127.0.0.1", port=0, dtype="fp32")
+    server, front = build_checkpoint_server(args, torch.float32, torch.device(DEV))
+    jobs = [("what a fine day it is today", 6), ("one two three four five six seven eight nine ten eleven twelve", 9), ("hello", 4)]
+
+    async def go():
+        await server.start()
+        front.start()
+        try:
+            return await asyncio.gather(*[_client_stream(f"http://127.0.0.1:{server.port}/v1", _payload(t, None, n)) for t, n in jobs])
+        finally:
+            front.stop()
+            await server.close()
+    got = asyncio.run(go())
+    assert front.error is None and front.n_admitted == len(jobs)
+    eng = OfflineInferenceEngine.from_checkpoint(str(tmp_path), torch.float32, DEV, max_running_requests=4, max_context=128, warm_up=False)
+    for (text, n_events, done), (prompt, n) in zip(got, jobs):
+        assert done and n_events == n + 1 and len(text.split()) == n
+        ids = server._token_request(parse(_payload(prompt, None, n))).token_ids
+        want = eng.generate([OfflineRequest(token_ids=ids, max_tokens=n)])[0].output_token_ids
+        assert text == "".join(server.tokenizer.decode(t) for t in want)
