@@ -100,7 +100,7 @@ class PemalornShape:
     hidden_size: int
     layers: List[PemalornLayer]
     norm_eps: float = 1e-5
-    taps: int = 1                     # taps of the input convolutions; 1 with no convolution tensors: none
+    taps: int = 0                     # taps of the input convolutions (one tap: h (1 + w)); 0: the design's layers have none
     side_dim: int = 0                 # per-layer slice of the token's second embedding; 0: no per-layer token input
     loop_start: int = 0
     loop_stop: int = 0
@@ -143,6 +143,8 @@ class PemalornShape:
                     raise ValueError(f"layer {i}: rot_dim must be even")
             else:
                 raise ValueError(f"layer {i}: unknown mixer type {m.type!r}")
+            if self.taps < 0:
+                raise ValueError("canon.taps must not be negative")
             if l.mlp is not None and (l.mlp.experts < 1 or not 1 <= l.mlp.top <= l.mlp.experts + l.mlp.identity):
                 raise ValueError(f"layer {i}: at least one expert with tensors, and top within the router's outputs")
         # a layer run's piece of a sequence's state: the last taps - 1 inputs of its convolutions
@@ -150,7 +152,8 @@ class PemalornShape:
 
     @property
     def state_piece_floats(self) -> int:
-        return (self.taps - 1) * self.hidden_size if self.taps > 1 else 0
+        # (one tap keeps nothing, but its kernel is handed a piece like the others: a row of `width` nobody reads)
+        return max(self.taps - 1, 1) * self.hidden_size if self.taps >= 1 else 0
 
     def state_piece(self, run: int) -> int:
         return run * self.state_piece_floats
@@ -202,7 +205,7 @@ class PemalornShape:
         if loop and int(loop["stop"]) <= int(loop["start"]):
             loop = None               # a span without layers: nothing runs twice, and no pass is ever entered
         return cls(vocab_size=int(cfg["vocab"]), hidden_size=int(cfg["width"]), layers=layers,
-                   norm_eps=float((cfg.get("norm") or {}).get("eps", 1e-5)), taps=int((cfg.get("canon") or {}).get("taps", 1)),
+                   norm_eps=float((cfg.get("norm") or {}).get("eps", 1e-5)), taps=int((cfg.get("canon") or {}).get("taps", 0)),
                    side_dim=int((cfg.get("token_side") or {}).get("dim", 0)),
                    loop_start=int(loop["start"]) if loop else 0, loop_stop=int(loop["stop"]) if loop else 0,
                    loop_times=int(loop.get("times", 1)) if loop else 1, has_loop=bool(loop))
@@ -227,7 +230,7 @@ class PemalornShape:
             out.append({"type": m.type, "mixer": mixer, "mlp": mlp})
         cfg = {"architecture": ARCHITECTURE, "vocab": self.vocab_size, "width": self.hidden_size,
                "norm": {"eps": self.norm_eps}, "layers": out}
-        if self.taps > 1:
+        if self.taps >= 1:
             cfg["canon"] = {"taps": self.taps}
         if self.side_dim:
             cfg["token_side"] = {"dim": self.side_dim}
@@ -261,7 +264,7 @@ def tensor_shapes(shape: PemalornShape) -> Dict[str, tuple]:
             for e in range(f.experts):
                 out.update({p + f"mlp.e{e}.gate": (f.ff, W), p + f"mlp.e{e}.up": (f.ff, W), p + f"mlp.e{e}.down": (W, f.ff)})
             out.update({p + "mlp.router": (f.experts + f.identity, W), p + "mlp.correction": (f.experts + f.identity,)})
-        if shape.taps > 1:
+        if shape.taps >= 1:
             out[p + "canon1"] = (W, shape.taps)
             if l.mlp is not None:
                 out[p + "canon2"] = (W, shape.taps)

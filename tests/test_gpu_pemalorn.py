@@ -54,11 +54,16 @@ def _shape(kind: str):
             L(lat(2, 64, 16, 64, 112, 32, 0.1, None, R(16, 500.0)), None),
             L(att(4, 4, 32, 64, 0.15, None, R(32, 10000.0, 8.0, 32.0, 8.0, 2.0)), E(3, 1, 2, 48))],
             norm_eps=1e-6, taps=5)
-    if kind == "plain":       # no convolutions (no state slots), no token input, one pass through a whole-model loop
+    if kind == "plain":       # convolutions of ONE tap (nothing to carry), no token input, one pass through a whole-model loop
         return PemalornShape(33, 48, [
             L(att(6, 3, 8, 8, 0.35, 9, R(8, 100.0)), E(2, 0, 2, 20)),
             L(lat(2, 12, 4, 20, 24, 12, 0.3, None, R(4, 100.0)), E(1, 1, 1, 32))],
             norm_eps=1e-5, taps=1, loop_start=0, loop_stop=2, loop_times=1, has_loop=True)
+    if kind == "bare":        # no convolutions at all (no state slots), no token input, no loop
+        return PemalornShape(33, 48, [
+            L(lat(2, 12, 4, 20, 24, 12, 0.3, 13, R(4, 100.0)), E(3, 1, 2, 32)),
+            L(att(6, 2, 8, 12, 0.35, None, R(4, 100.0)), None)],
+            norm_eps=1e-5)
     raise KeyError(kind)
 
 
@@ -417,7 +422,7 @@ def test_router_with_correction_plain_weights_and_identity_experts(E, I, top, W_
 
 
 # ------------------------------------------------------------------------------------------------ the model in the engine
-@pytest.mark.parametrize("kind", ["mix", "odd", "wide", "plain"])
+@pytest.mark.parametrize("kind", ["mix", "odd", "wide", "plain", "bare"])
 def test_whole_prompts_match_the_oracle_layer_by_layer(kind):
     shape = _shape(kind)
     W = _weights(shape, seed=11)
@@ -446,11 +451,13 @@ def test_specs_the_engine_reads():
     assert [r[0] for r in m.shape.runs] == [0, 1, 2, 1, 2, 1, 2, 3] and [r[2] for r in m.shape.runs] == [False, True, False, True, False, True, False, False]
     assert m.shape.run_plane == [0, 2, 3, 5, 6, 8, 9, 11] and m.cache_spec() == {"n_layers": 12, "n_tokens": 1, "n_heads": 1, "head_size": 48}
     assert m.state_spec() == {"rows": 1, "width": 8 * 2 * 64} and m.shape.state_piece(3) == 3 * 128
-    assert p.state_spec() is None and p.cache_spec()["n_layers"] == 3
+    assert p.state_spec() == {"rows": 1, "width": 2 * 48} and p.cache_spec()["n_layers"] == 3
+    b = _model(_shape("bare"), _weights(_shape("bare")), torch.float32).language_model
+    assert b.state_spec() is None and "l0.canon1" not in b.shape.to_config() and b.shape.to_config().get("canon") is None
     assert m.shape.to_config() == type(m.shape).from_config(m.shape.to_config()).to_config()
 
 
-@pytest.mark.parametrize("kind", ["mix", "odd", "wide", "plain"])
+@pytest.mark.parametrize("kind", ["mix", "odd", "wide", "plain", "bare"])
 def test_decoding_token_by_token_and_portions_of_every_size_equal_the_whole_prompt(kind):
     shape = _shape(kind)
     W = _weights(shape, seed=13)

@@ -58,6 +58,8 @@ def test_configurations_without_loop_convolutions_or_token_input():
     names = tensor_shapes(sh)
     assert not any(k.startswith(("loop.", "side.")) or "canon" in k or ".side." in k for k in names)
     assert sh.to_config() == cfg
+    one = PemalornShape.from_config(_config(canon={"taps": 1}))          # one tap is still a convolution: h (1 + w)
+    assert tensor_shapes(one)["l0.canon1"] == (24, 1) and one.state_floats == 6 * 24 and one.to_config()["canon"] == {"taps": 1}
     whole = PemalornShape.from_config(_config(loop={"start": 0, "stop": 4, "times": 1}))      # one pass still enters through the loop's input
     assert [r[2] for r in whole.runs] == [True, False, False, False]
     empty = PemalornShape.from_config(_config(loop={"start": 3, "stop": 3, "times": 4}))      # a span without layers is no loop
